@@ -1,0 +1,158 @@
+/*
+ * libshainet_hip_kernels.so: C ABI of the MI355X (gfx950) attention hot path
+ * of SHAInet's LlamaBlock: Q/K/V bias, Qwen3 per-head QK-RMSNorm, half-split
+ * RoPE, KV-cache append and causal grouped-query attention (decode and prefill),
+ * all fp32, all on the device.
+ *
+ * Plain pointers and ints only; every function returns an int status
+ * (0 = ok) unless it mirrors a reference symbol that returns void.  A failing
+ * call leaves a message for shainet_hip_last_error().
+ *
+ * Threading: one caller at a time per context (the reference serialises its
+ * callers the same way, examples/openai_server.cr:57-62).  Work is issued on the
+ * context's own HIP stream; calls that take host pointers return with the result
+ * in place, calls that take device pointers are asynchronous until
+ * shainet_attn_sync().
+ */
+#ifndef SHAINET_HIP_ATTN_H
+#define SHAINET_HIP_ATTN_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SHAINET_HIP_OK 0
+#define SHAINET_HIP_ERR_ARGUMENT 1 /* the Crystal layer raises ArgumentError */
+#define SHAINET_HIP_ERR_RUNTIME 2  /* a HIP runtime call or a launch failed */
+#define SHAINET_HIP_ERR_ALLOC 3    /* device allocation failed: Crystal runs GC.collect and retries (cuda.cr:124-140) */
+#define SHAINET_HIP_ERR_CAPACITY 4 /* the cache cannot hold the appended rows */
+
+#define SHAINET_HIP_MEM_HOST 0   /* q,k,v,out are host pointers; the call is synchronous */
+#define SHAINET_HIP_MEM_DEVICE 1 /* q,k,v,out are device pointers; the call is asynchronous */
+
+#define SHAINET_HIP_MAX_BATCH 64 /* sequences per shainet_attn_forward call */
+
+/* Message of the last failing call on this thread.  Replaces the reference's
+ * printf of cudaGetLastError (src/shainet/native/cuda_kernels.cu:722-725, 821-824). */
+const char *shainet_hip_last_error(void);
+
+/* 1 when a gfx950 device is visible and usable, else 0.  The counterpart of
+ * CUDA.fully_available? (src/shainet/cuda.cr:63-83, 111-122, 778-780). */
+int shainet_hip_available(void);
+
+/* ---- entry points with the reference's own names and signatures ----------- */
+
+/* Scatter the staged new rows into a [num_kv_heads, capacity, head_dim] cache
+ * at start_pos.  staging = K chunks (kv-head major, each new_tokens*head_dim)
+ * then V chunks, K already rotated.  Same symbol, arguments and layout as
+ * src/shainet/native/cuda_kernels.cu:713-726 (bound at src/shainet/cuda.cr:838-861).
+ * Runs on the default stream, like the reference. */
+void kv_cache_append_f32(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
+                         int num_kv_heads, int head_dim, int capacity);
+
+/* Causal GQA attention of new_tokens rotated query rows over the device cache.
+ * Same symbol, arguments and layouts as src/shainet/native/cuda_kernels.cu:808-825
+ * (bound at src/shainet/cuda.cr:866-891).  `ws` is accepted and ignored: scores
+ * never leave the chip.  Runs on the default stream, like the reference. */
+void attention_kv_f32(const float *q, const float *kc, const float *vc, float *out, float *ws,
+                      int new_tokens, int start_pos, int num_heads, int heads_per_kv, int head_dim,
+                      int capacity, float scale);
+
+/* ---- fused, batched entry points ------------------------------------------ */
+
+typedef struct shainet_attn_ctx shainet_attn_ctx;
+typedef struct shainet_kv_cache shainet_kv_cache;
+
+/* The attention parameters of one LlamaBlock (src/shainet/transformer/llama_block.cr:10-28,
+ * 73-108).  rope_freqs: NULL or head_dim/2 inverse frequencies that override
+ * theta^(-2i/head_dim) (llama_block.cr:669-675).  q_norm/k_norm: NULL or a
+ * weight vector with its length; a length other than head_dim is an argument
+ * error, as in llama_block.cr:618.  qk_norm_eps is the block's eps (llama_block.cr:92).
+ * max_positions sizes the cos/sin table (it grows on demand). */
+int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads, int head_dim,
+                        double rope_theta, const float *rope_freqs, const float *q_norm, int q_norm_len,
+                        const float *k_norm, int k_norm_len, double qk_norm_eps, int max_positions);
+
+/* Optional Q/K/V projection biases, added to the incoming rows before QK-norm
+ * (llama_block.cr:257-259, 585-601).  NULL clears one.  A length that is not
+ * num_heads*head_dim (q) or num_kv_heads*head_dim (k, v) is an argument error. */
+int shainet_attn_set_bias(shainet_attn_ctx *ctx, const float *b_q, int b_q_len, const float *b_k,
+                          int b_k_len, const float *b_v, int b_v_len);
+
+int shainet_attn_destroy(shainet_attn_ctx *ctx);
+
+/* Wait for everything issued on the context's stream. */
+int shainet_attn_sync(shainet_attn_ctx *ctx);
+
+/* The context's hipStream_t, for callers that enqueue their own work around it. */
+void *shainet_attn_stream(shainet_attn_ctx *ctx);
+
+/* Issue the context's work on a caller-owned hipStream_t instead (NULL = the
+ * default stream, which is what the reference uses throughout).  The context's
+ * own stream is kept and restored by passing the value shainet_attn_stream()
+ * returned before the first call of this function. */
+int shainet_attn_set_stream(shainet_attn_ctx *ctx, void *stream);
+
+/* Copy of the inverse frequencies in use (head_dim/2 floats, host). */
+int shainet_attn_inv_freq(shainet_attn_ctx *ctx, float *out);
+
+/* A device-resident fp32 KV cache for `batch` independent sequences, each
+ * [num_kv_heads, capacity, head_dim] for K and for V: the reference's device
+ * layout (llama_block.cr:50-56, 497-520) with a leading sequence index.  The
+ * device copy is the cache of record; there is no host mirror. */
+int shainet_kv_cache_create(shainet_kv_cache **out, shainet_attn_ctx *ctx, int batch, int capacity);
+int shainet_kv_cache_destroy(shainet_kv_cache *cache);
+
+/* LlamaBlock#clear_cache! (llama_block.cr:116-122): lengths go to 0, memory is
+ * kept, stale rows are overwritten before they can become visible.  seq < 0
+ * clears every sequence. */
+int shainet_kv_cache_clear(shainet_kv_cache *cache, int seq);
+
+/* Number of cached positions of one sequence (@cache_len, llama_block.cr:48), or -1. */
+int shainet_kv_cache_len(const shainet_kv_cache *cache, int seq);
+int shainet_kv_cache_capacity(const shainet_kv_cache *cache);
+
+/* Grow every sequence's capacity to at least `capacity`, keeping contents
+ * (the job of ensure_gpu_cache!, llama_block.cr:497-520, without the host mirror). */
+int shainet_kv_cache_reserve(shainet_kv_cache *cache, int capacity);
+
+/* Device base pointers of the K and V arrays: [batch][num_kv_heads][capacity][head_dim]. */
+float *shainet_kv_cache_k(shainet_kv_cache *cache);
+float *shainet_kv_cache_v(shainet_kv_cache *cache);
+
+/* Replace one sequence's contents with n rows per kv head, K already rotated:
+ * k_rows, v_rows are [num_kv_heads][n][head_dim] (host when mem == HOST).  The
+ * reference has no cache setter (its cache is private state, llama_block.cr:46-48);
+ * benchmarks that start from a pre-filled cache and tests need one. */
+int shainet_kv_cache_fill(shainet_kv_cache *cache, int seq, const float *k_rows, const float *v_rows, int n,
+                          int mem);
+
+/* Copy rows [pos0, pos0+n) of one kv head of one sequence to host buffers
+ * ([n][head_dim] each; either may be NULL).  For tests of the cache contract. */
+int shainet_kv_cache_read(shainet_kv_cache *cache, int seq, int kv_head, int pos0, int n, float *k_out,
+                          float *v_out);
+
+/* attention_cached_cpu from the projections' outputs to the head loop's output
+ * (llama_block.cr:256-296), for n_seqs sequences at once, entirely on the device:
+ * bias, QK-norm, RoPE with positions cache_len .. cache_len+new_tokens-1, append
+ * of the rotated K rows and the V rows, causal GQA attention over the cache.
+ *   seq_ids[n_seqs]     cache slots taking part, distinct (NULL = 0..n_seqs-1)
+ *   new_tokens[n_seqs]  rows appended per sequence (>= 1)
+ *   q   [sum new_tokens, num_heads*head_dim]      rows of sequence seq_ids[0] first
+ *   k,v [sum new_tokens, num_kv_heads*head_dim]
+ *   out [sum new_tokens, num_heads*head_dim]
+ * Each sequence's length grows by its new_tokens.  SHAINET_HIP_ERR_CAPACITY (and
+ * nothing appended) if a sequence would outgrow the capacity. */
+int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const int *seq_ids,
+                         const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
+                         float *out, int mem);
+
+/* Copy of the rotated query rows of the last shainet_attn_forward call
+ * ([sum new_tokens, num_heads*head_dim], host): lets a test check RoPE positions
+ * and QK-norm of Q exactly (llama_block.cr:332-344). */
+int shainet_attn_last_q_rot(shainet_attn_ctx *ctx, float *out, int rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

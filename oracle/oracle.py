@@ -48,6 +48,8 @@ def lib():
         L.orc_block_v_cache.restype = _f32p
         L.orc_block_fill_cache.argtypes = [C.c_void_p, _f32p, _f32p, C.c_int]
         L.orc_inv_freq.argtypes = [C.c_void_p, _f32p]
+        L.orc_rotate_q.argtypes = [C.c_void_p, _f32p, _f32p, C.c_int, C.c_int]
+        L.orc_rotate_q.restype = None
         L.orc_scale.argtypes = [C.c_void_p]
         L.orc_scale.restype = C.c_float
         L.orc_head_rmsnorm.argtypes = [C.c_void_p, _f32p, C.c_int, C.c_int, _f32p, C.c_int]
@@ -165,21 +167,26 @@ class Block:
     def scale(self):
         return lib().orc_scale(self._h)
 
-    def attention_cached_qkv(self, q, k, v, threads=1):
+    def attention_cached_qkv(self, q, k, v, threads=1, keep_q_rot=False):
         """llama_block.cr:256-296 on projected rows; returns output [T, q_dim].
 
         threads > 1 runs disjoint query-head ranges concurrently; every head's
-        arithmetic is unchanged."""
+        arithmetic is unchanged.  keep_q_rot stores the rotated query rows
+        (llama_block.cr:332-344) in self.last_q_rot."""
         q, k, v = (np.array(a, dtype=np.float32, order="C") for a in (q, k, v))
         T = q.shape[0]
         assert q.shape == (T, self.q_dim) and k.shape == (T, self.kv_dim) and v.shape == (T, self.kv_dim)
         out = np.empty((T, self.q_dim), np.float32)
-        if threads <= 1:
+        if threads <= 1 and not keep_q_rot:
             _check(lib().orc_block_attention_cached_qkv(self._h, _p(q), _p(k), _p(v), T, _p(out)))
             return out
         start = C.c_int(0)
         _check(lib().orc_block_prepare_append(self._h, _p(q), _p(k), _p(v), T, C.byref(start)))
+        if keep_q_rot:
+            self.last_q_rot = np.empty_like(q)
+            lib().orc_rotate_q(self._h, _p(q), _p(self.last_q_rot), T, start.value)
         total, scale, H = self.cache_len, self.scale(), self.num_heads
+        threads = max(1, threads)
         threads = min(threads, H)
         bounds = [H * i // threads for i in range(threads + 1)]
 

@@ -390,6 +390,27 @@ void orc_attention_heads_cpu(const OrcBlock *b, const float *q_full, float *outp
   free(q_rot); free(scores); free(out);
 }
 
+/* The query rotation alone (llama_block.cr:332-344), for every head and row of
+ * q_full [T,q_dim] (after bias and QK-norm): lets a test compare the device's
+ * rotated rows bit for bit. */
+void orc_rotate_q(const OrcBlock *b, const float *q_full, float *q_rot, int new_tokens, int start_pos) {
+  int hd = b->head_dim, half = hd / 2, dm = b->q_dim;
+  memset(q_rot, 0, sizeof(float) * (size_t)new_tokens * dm);
+  for (int h = 0; h < b->num_heads; ++h)
+    for (int i = 0; i < new_tokens; ++i) {
+      int pos = start_pos + i;
+      size_t qrow = (size_t)i * dm + (size_t)h * hd;
+      for (int idx = 0; idx < half; ++idx) {
+        float freq = inv_freq(b, idx);
+        float angle = (float)pos * freq;
+        float c = cosf(angle), s = sinf(angle);
+        float x0 = q_full[qrow + idx], x1 = q_full[qrow + idx + half];
+        q_rot[qrow + idx] = x0 * c - x1 * s;
+        q_rot[qrow + idx + half] = x1 * c + x0 * s;
+      }
+    }
+}
+
 /* scale : llama_block.cr:249. */
 float orc_scale(const OrcBlock *b) { return (float)(1.0 / sqrt((double)b->head_dim)); }
 

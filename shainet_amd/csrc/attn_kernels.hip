@@ -1,0 +1,550 @@
+// Causal grouped-query attention over the device KV cache for gfx950 (CDNA4).
+//
+// Three kernels replace attention_heads_cpu (llama_block.cr:302-401) and the
+// reference's attention_kv_kernel (cuda_kernels.cu:734-806):
+//
+//   decode_splitk_kernel  one new row per sequence.  Split-K over the cached
+//       positions: every wavefront streams 16-key tiles of K and V straight from
+//       HBM into MFMA operands (v_mfma_f32_16x16x4_f32, the g query heads of a
+//       GQA group are the tile's columns, so K and V are read once per group),
+//       keeps an online softmax, and the four wavefronts of a workgroup merge
+//       their (max, sum, O) through LDS.  A second small kernel merges the
+//       workgroups of one sequence.
+//   prefill_mfma_kernel   many new rows.  Query rows and the heads of a group
+//       are flattened into "virtual rows"; a wavefront owns 32 of them, a
+//       workgroup 128.  K/V tiles of 32 keys are staged through LDS (double
+//       buffered) and consumed by v_mfma_f32_32x32x2_f32.
+//   generic_attn_kernel   any head_dim; one wavefront per (row, head).  Used for
+//       head dims other than 64 and 128.
+//
+// All three compute S^T = K Q^T so that the probabilities come out of the MFMA
+// accumulator already laid out as the B operand of O^T = V^T P^T: no transpose,
+// no LDS round trip for P.  The contraction index of an MFMA may be visited in
+// any order as long as A and B agree, which lets every lane fetch 16-byte
+// pieces of K rows.
+#include "attn_kernels.hpp"
+
+#include <math.h>
+
+namespace shainet {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ int find_seq(const SeqTable &st, int item, const int *off) {
+  int s = 0;
+  while (s + 1 < st.n_seqs && item >= off[s + 1]) ++s;
+  return s;
+}
+
+// ---------------------------------------------------------------------------
+// Decode: split-K, one new row per sequence.
+//
+// MFMA 16x16x4 operand layout (lane l): A[m = l%16][k = l/16], B[k = l/16][n = l%16],
+// D[m = 4*(l/16) + r][n = l%16] for accumulator register r = 0..3.
+//   scores:  D = S^T, m = key within the tile, n = query head within the group.
+//            K-step s of lane group j = l/16 covers d = 16*(s/4) + 4*j + s%4, so
+//            a lane fetches K as float4 at offsets 16*i + 4*j of its key row.
+//   output:  D = O^T tile t, m = d index, n = head; the contraction runs over the
+//            tile's keys, k-step r of lane group j is key 4*j + r, which is exactly
+//            where accumulator register r of S^T lives.  Row m of tile t is
+//            d = NT*m + t, so a lane fetches NT consecutive floats of a V row.
+template <int HD>
+__global__ __launch_bounds__(256) void decode_splitk_kernel(const float *__restrict__ q_rot,
+                                                            const float *__restrict__ kc,
+                                                            const float *__restrict__ vc,
+                                                            float *__restrict__ out,
+                                                            float *__restrict__ part_o,
+                                                            float *__restrict__ part_ml, SeqTable st,
+                                                            Shape sh, int chunk, float c) {
+  constexpr int NT = HD / 16;  // float4 loads per lane per K tile; d tiles of the output
+  extern __shared__ float smem[];
+  const int item = blockIdx.x, kvh = blockIdx.y;
+  const int s = find_seq(st, item, st.work_off);
+  const int ci = item - st.work_off[s];
+  const int n_chunks = st.work_off[s + 1] - st.work_off[s];
+  const int L = st.start_pos[s] + 1;  // visible keys of the one new row
+  const int k_begin = ci * chunk;
+  const int k_end = min(L, k_begin + chunk);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int g = sh.g;
+  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
+  const float *kbase = kc + head_base;
+  const float *vbase = vc + head_base;
+  const int token = st.tok_off[s];
+
+  float qr[HD / 4];
+  {
+    const float *qp = q_rot + ((long long)token * sh.H + kvh * g + (col < g ? col : 0)) * HD + 4 * j;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      f32x4 t = *(const f32x4 *)(qp + 16 * i);
+      if (col >= g) t = f32x4{0.f, 0.f, 0.f, 0.f};
+      qr[4 * i + 0] = t.x;
+      qr[4 * i + 1] = t.y;
+      qr[4 * i + 2] = t.z;
+      qr[4 * i + 3] = t.w;
+    }
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = k_begin + wave * 16; kb < k_end; kb += 64) {
+    // rows past the end are clamped to the last valid row: finite data, weight 0
+    const float *kp = kbase + (long long)min(kb + col, L - 1) * HD + 4 * j;
+    f32x4 kr[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) kr[i] = *(const f32x4 *)(kp + 16 * i);
+    float vr[4][NT];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float *vp = vbase + (long long)min(kb + 4 * j + r, L - 1) * HD + NT * col;
+#pragma unroll
+      for (int i = 0; i < NT / 4; ++i) {
+        f32x4 t = *(const f32x4 *)(vp + 4 * i);
+        vr[r][4 * i + 0] = t.x;
+        vr[r][4 * i + 1] = t.y;
+        vr[r][4 * i + 2] = t.z;
+        vr[r][4 * i + 3] = t.w;
+      }
+    }
+
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].x, qr[4 * i + 0], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].y, qr[4 * i + 1], s1, 0, 0, 0);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].z, qr[4 * i + 2], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].w, qr[4 * i + 3], s1, 0, 0, 0);
+    }
+    float sv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sv[r] = (kb + 4 * j + r < k_end) ? s0[r] + s1[r] : -INFINITY;
+    float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mnew = fmaxf(m, mx);  // finite: key kb is valid
+    const float alpha = fast_exp2((m - mnew) * c);
+    float p[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) p[r] = fast_exp2((sv[r] - mnew) * c);
+    l = l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
+    m = mnew;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) o[t] *= alpha;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) o[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[r][t], p[r], o[t], 0, 0, 0);
+  }
+
+  // merge the four wavefronts through LDS: sm_o[wave][col][d], sm_m/sm_l[wave][col]
+  l += __shfl_xor(l, 16);
+  l += __shfl_xor(l, 32);
+  float *sm_o = smem;
+  float *sm_m = smem + 4 * g * HD;
+  float *sm_l = sm_m + 4 * g;
+  if (col < g) {
+    float *dst = sm_o + (wave * g + col) * HD;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) dst[NT * (4 * j + r) + t] = o[t][r];
+    if (j == 0) {
+      sm_m[wave * g + col] = m;
+      sm_l[wave * g + col] = l;
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < g * HD; idx += 256) {
+    const int cc = idx / HD, d = idx - cc * HD;
+    float mm = sm_m[cc];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w * g + cc]);
+    float acc = 0.f, ls = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = fast_exp2((sm_m[w * g + cc] - mm) * c);  // 0 for a wavefront that saw no key
+      acc += f * sm_o[(w * g + cc) * HD + d];
+      ls += f * sm_l[w * g + cc];
+    }
+    const int h = kvh * g + cc;
+    if (n_chunks == 1) {
+      out[((long long)token * sh.H + h) * HD + d] = acc / ls;
+    } else {
+      const long long pi = ((long long)item * sh.KV + kvh) * g + cc;
+      part_o[pi * HD + d] = acc;
+      if (d == 0) {
+        part_ml[2 * pi] = mm;
+        part_ml[2 * pi + 1] = ls;
+      }
+    }
+  }
+}
+
+// Merge the split-K partials of one (sequence, head): online-softmax combine.
+__global__ void decode_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                      float *__restrict__ out, SeqTable st, Shape sh, float c) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int first = st.work_off[s], n = st.work_off[s + 1] - first;
+  if (n <= 1) return;  // written by the split kernel itself
+  const int kvh = h / sh.g, cc = h - kvh * sh.g;
+  const int hd = sh.hd;
+  float mm = -INFINITY;
+  for (int i = 0; i < n; ++i) mm = fmaxf(mm, part_ml[2 * ((((long long)(first + i)) * sh.KV + kvh) * sh.g + cc)]);
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float acc = 0.f, ls = 0.f;
+    for (int i = 0; i < n; ++i) {
+      const long long pi = (((long long)(first + i)) * sh.KV + kvh) * sh.g + cc;
+      const float f = fast_exp2((part_ml[2 * pi] - mm) * c);
+      acc += f * part_o[pi * hd + d];
+      ls += f * part_ml[2 * pi + 1];
+    }
+    out[((long long)st.tok_off[s] * sh.H + h) * hd + d] = acc / ls;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Prefill: MFMA 32x32x2, K/V tiles staged through LDS.
+//
+// Virtual row v of a (sequence, kv head): query row v / g, head kvh*g + v % g.
+// MFMA 32x32x2 layout (lane l): A[m = l%32][k = l/32], B[k = l/32][n = l%32],
+// D[m = 8*(r/4) + 4*(l/32) + r%4][n = l%32] for accumulator register r = 0..15.
+//   scores:  m = key within the tile, n = virtual row; k-step s of lane half
+//            j = l/32 covers d = 8*(s/4) + 4*j + s%4 (float4 pieces of a K row).
+//   output:  tile t, m = d index (d = NT*m + t), contraction over the tile's keys in
+//            the order the score accumulator holds them.
+template <int HD>
+__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__restrict__ q_rot,
+                                                              const float *__restrict__ kc,
+                                                              const float *__restrict__ vc,
+                                                              float *__restrict__ out, SeqTable st, Shape sh,
+                                                              float c) {
+  constexpr int NK4 = HD / 8;   // float4 pieces of a K row per lane
+  constexpr int NT = HD / 32;   // d tiles of the output
+  constexpr int KSTR = HD + 4;  // padded K row stride in LDS: conflict-free 16-byte reads down a column
+  constexpr int LD4 = HD / 32;  // float4 per thread to stage one K (or V) tile
+  __shared__ float Ks[2][32 * KSTR];
+  __shared__ float Vs[2][32 * HD];
+
+  const int item = blockIdx.x, kvh = blockIdx.y;
+  const int s = find_seq(st, item, st.work_off);
+  const int nblk = st.work_off[s + 1] - st.work_off[s];
+  const int vb = nblk - 1 - (item - st.work_off[s]);  // longest rows first
+  const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
+  const int L = S + T, VR = T * g;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, j = lane >> 5;
+  const int v0 = vb * 128 + wave * 32;
+  const bool wave_active = v0 < VR;
+  const int my_v = v0 + n;
+  const bool valid = my_v < VR;
+  const int row = valid ? my_v / g : T - 1;
+  const int hg = valid ? my_v - row * g : 0;
+  const int lim = S + row;                                            // last visible key of this lane's row
+  const int wave_lo = S + (wave_active ? v0 / g : 0);                 // smallest lim in the wavefront
+  const int wave_hi = wave_active ? S + min(v0 + 31, VR - 1) / g : -1;  // largest
+  const int wg_hi = S + min(vb * 128 + 127, VR - 1) / g;
+  const int n_tiles = wg_hi / 32 + 1;
+  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
+  const float *kbase = kc + head_base;
+  const float *vbase = vc + head_base;
+  const long long qo_off = ((long long)(st.tok_off[s] + row) * sh.H + kvh * g + hg) * HD;
+
+  float qr[HD / 2];
+  {
+    const float *qp = q_rot + qo_off + 4 * j;
+#pragma unroll
+    for (int i = 0; i < NK4; ++i) {
+      f32x4 t = *(const f32x4 *)(qp + 8 * i);
+      if (!valid) t = f32x4{0.f, 0.f, 0.f, 0.f};
+      qr[4 * i + 0] = t.x;
+      qr[4 * i + 1] = t.y;
+      qr[4 * i + 2] = t.z;
+      qr[4 * i + 3] = t.w;
+    }
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x16 o[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
+
+  f32x4 stage_k[LD4], stage_v[LD4];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int u = 0; u < LD4; ++u) {
+      const int idx = threadIdx.x + 256 * u;
+      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
+      const long long src = (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4;
+      stage_k[u] = *(const f32x4 *)(kbase + src);
+      stage_v[u] = *(const f32x4 *)(vbase + src);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < LD4; ++u) {
+      const int idx = threadIdx.x + 256 * u;
+      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
+      *(f32x4 *)&Ks[buf][r * KSTR + 4 * c4] = stage_k[u];
+      *(f32x4 *)&Vs[buf][r * HD + 4 * c4] = stage_v[u];
+    }
+  };
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < n_tiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < n_tiles) load_tile(kt + 1);
+    if (kt * 32 <= wave_hi) {
+      f32x16 sacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+      const float *kl = &Ks[buf][n * KSTR + 4 * j];
+#pragma unroll
+      for (int i = 0; i < NK4; ++i) {
+        const f32x4 kv = *(const f32x4 *)(kl + 8 * i);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[4 * i + 0], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[4 * i + 1], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[4 * i + 2], sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[4 * i + 3], sacc, 0, 0, 0);
+      }
+      if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kt * 32 + 8 * (r >> 2) + 4 * j + (r & 3);
+          if (key > lim) sacc[r] = -INFINITY;
+        }
+      }
+      float mx = sacc[0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mnew = fmaxf(m, mx);  // finite from tile 0 on: key 0 is visible to every row
+      const float alpha = fast_exp2((m - mnew) * c);
+      const float mc = mnew * c;
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sacc[r] = fast_exp2(sacc[r] * c - mc);
+        psum += sacc[r];
+      }
+      l = l * alpha + psum;
+      if (__any(mnew != m)) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+      }
+      m = mnew;
+      const float *vl = &Vs[buf][4 * j * HD + NT * n];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float *vp = vl + (8 * (r >> 2) + (r & 3)) * HD;
+        if constexpr (NT == 2) {
+          const float2 vv = *(const float2 *)vp;
+          o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, sacc[r], o[0], 0, 0, 0);
+          o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, sacc[r], o[1], 0, 0, 0);
+        } else {
+          const f32x4 vv = *(const f32x4 *)vp;
+          o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, sacc[r], o[0], 0, 0, 0);
+          o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, sacc[r], o[1], 0, 0, 0);
+          o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.z, sacc[r], o[2], 0, 0, 0);
+          o[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.w, sacc[r], o[3], 0, 0, 0);
+        }
+      }
+    }
+    if (kt + 1 < n_tiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  l += __shfl_xor(l, 32);
+  if (valid) {
+    const float inv = 1.0f / l;
+    float *op = out + qo_off;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int d = NT * (8 * (r >> 2) + 4 * j + (r & 3));
+      if constexpr (NT == 2) {
+        *(float2 *)(op + d) = float2{o[0][r] * inv, o[1][r] * inv};
+      } else {
+        *(f32x4 *)(op + d) = f32x4{o[0][r] * inv, o[1][r] * inv, o[2][r] * inv, o[3][r] * inv};
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Any head_dim up to 256: one wavefront per (row, head), lane = key for the
+// scores, lane = d for the output.
+__global__ __launch_bounds__(64) void generic_attn_kernel(const float *__restrict__ q_rot,
+                                                          const float *__restrict__ kc,
+                                                          const float *__restrict__ vc,
+                                                          float *__restrict__ out, SeqTable st, Shape sh,
+                                                          float scale) {
+  extern __shared__ float smem[];
+  const int hd = sh.hd;
+  float *q_s = smem, *p_s = smem + hd;
+  const int token = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int s = find_seq(st, token, st.tok_off);
+  const int visible = st.start_pos[s] + (token - st.tok_off[s]) + 1;
+  const int kvh = h / sh.g;
+  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * hd;
+  const float *kbase = kc + head_base, *vbase = vc + head_base;
+  const long long qo = ((long long)token * sh.H + h) * hd;
+  for (int d = lane; d < hd; d += 64) q_s[d] = q_rot[qo + d];
+  __syncthreads();
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  for (int j0 = 0; j0 < visible; j0 += 64) {
+    const int jj = j0 + lane;
+    float sv = -INFINITY;
+    if (jj < visible) {
+      const float *kr = kbase + (long long)jj * hd;
+      float dot = 0.f;
+      for (int d = 0; d < hd; ++d) dot += q_s[d] * kr[d];
+      sv = dot * scale;
+    }
+    float mx = sv;
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    const float mnew = fmaxf(m, mx);
+    const float alpha = expf(m - mnew);
+    const float p = expf(sv - mnew);
+    float ps = p;
+    for (int o = 32; o > 0; o >>= 1) ps += __shfl_xor(ps, o);
+    l = l * alpha + ps;
+    m = mnew;
+    p_s[lane] = p;
+    __syncthreads();
+    const int cnt = min(64, visible - j0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int d = lane + 64 * u;
+      if (d < hd) {
+        float a = acc[u] * alpha;
+        for (int t = 0; t < cnt; ++t) a += p_s[t] * vbase[(long long)(j0 + t) * hd + d];
+        acc[u] = a;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int d = lane + 64 * u;
+    if (d < hd) out[qo + d] = acc[u] / l;
+  }
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+}  // namespace
+
+Path choose_path(const SeqTable &st, const Shape &sh) {
+  if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
+  bool all_single = true;
+  for (int s = 0; s < st.n_seqs; ++s) all_single = all_single && st.n_new[s] == 1;
+  if (all_single && sh.g <= 16) return Path::kDecodeSplitK;
+  return Path::kPrefillMfma;
+}
+
+int choose_decode_chunk(const SeqTable &st, const Shape &sh) {
+  long long keys = 0;
+  for (int s = 0; s < st.n_seqs; ++s) keys += st.start_pos[s] + 1;
+  // aim for about eight workgroups per compute unit over the whole launch
+  long long chunk = (keys * sh.KV + 2047) / 2048;
+  chunk = (chunk + 63) / 64 * 64;
+  if (chunk < 64) chunk = 64;
+  if (chunk > 1024) chunk = 1024;
+  return (int)chunk;
+}
+
+int plan_work(SeqTable &st, const Shape &sh, Path path, int decode_chunk) {
+  st.work_off[0] = 0;
+  for (int s = 0; s < st.n_seqs; ++s) {
+    int items;
+    if (path == Path::kDecodeSplitK)
+      items = (st.start_pos[s] + 1 + decode_chunk - 1) / decode_chunk;
+    else if (path == Path::kPrefillMfma)
+      items = (st.n_new[s] * sh.g + 127) / 128;
+    else
+      items = st.n_new[s];
+    st.work_off[s + 1] = st.work_off[s] + items;
+  }
+  return st.work_off[st.n_seqs];
+}
+
+size_t decode_partial_floats(const Shape &sh, int items) {
+  return (size_t)items * sh.KV * sh.g * (sh.hd + 2);
+}
+
+static bool table_ok(const SeqTable &st, const Shape &sh) {
+  if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.H != sh.KV * sh.g) return false;
+  for (int s = 0; s < st.n_seqs; ++s)
+    if (st.n_new[s] < 1 || st.start_pos[s] < 0 || st.start_pos[s] + st.n_new[s] > sh.cap || st.slot[s] < 0)
+      return false;
+  return true;
+}
+
+hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
+                         const SeqTable &st, const Shape &sh, int items, int decode_chunk, float scale,
+                         hipStream_t stream) {
+  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || sh.g > 16 || decode_chunk % 64 || items < 1)
+    return hipErrorInvalidValue;
+  for (int s = 0; s < st.n_seqs; ++s)
+    if (st.n_new[s] != 1) return hipErrorInvalidValue;
+  float *part_o = partials;
+  float *part_ml = partials + (size_t)items * sh.KV * sh.g * sh.hd;
+  const float c = scale * kLog2e;
+  const size_t smem = (size_t)(4 * sh.g * sh.hd + 8 * sh.g) * sizeof(float);
+  dim3 grid((unsigned)items, (unsigned)sh.KV);
+  if (sh.hd == 64)
+    hipLaunchKernelGGL(decode_splitk_kernel<64>, grid, dim3(256), smem, stream, q_rot, kc, vc, out, part_o, part_ml,
+                       st, sh, decode_chunk, c);
+  else
+    hipLaunchKernelGGL(decode_splitk_kernel<128>, grid, dim3(256), smem, stream, q_rot, kc, vc, out, part_o,
+                       part_ml, st, sh, decode_chunk, c);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (items > st.n_seqs) {  // some sequence was split
+    hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)st.n_seqs, (unsigned)sh.H), dim3(sh.hd), 0, stream,
+                       part_o, part_ml, out, st, sh, c);
+    e = hipGetLastError();
+  }
+  return e;
+}
+
+hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
+                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream) {
+  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1) return hipErrorInvalidValue;
+  const float c = scale * kLog2e;
+  dim3 grid((unsigned)items, (unsigned)sh.KV);
+  if (sh.hd == 64)
+    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), 0, stream, q_rot, kc, vc, out, st, sh, c);
+  else
+    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), 0, stream, q_rot, kc, vc, out, st, sh, c);
+  return hipGetLastError();
+}
+
+hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
+                          const SeqTable &st, const Shape &sh, int total_tokens, float scale,
+                          hipStream_t stream) {
+  if (!table_ok(st, sh) || sh.hd < 1 || sh.hd > 256 || total_tokens < 1) return hipErrorInvalidValue;
+  const size_t smem = (size_t)(sh.hd + 64) * sizeof(float);
+  hipLaunchKernelGGL(generic_attn_kernel, dim3((unsigned)total_tokens, (unsigned)sh.H), dim3(64), smem, stream,
+                     q_rot, kc, vc, out, st, sh, scale);
+  return hipGetLastError();
+}
+
+}  // namespace shainet

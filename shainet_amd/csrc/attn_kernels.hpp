@@ -1,0 +1,65 @@
+// Launchers of the gfx950 attention kernels.  Device pointers only; every
+// launcher validates the shapes its kernel assumes and returns a hipError_t.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace shainet {
+
+constexpr int kMaxSeqs = 64;
+
+// Per-call description of the sequences taking part, passed to kernels by value
+// (it lives in the kernel-argument segment, so no copy to the device is needed).
+struct SeqTable {
+  int n_seqs;
+  int slot[kMaxSeqs];          // cache slot of sequence s
+  int start_pos[kMaxSeqs];     // cached positions before this call
+  int n_new[kMaxSeqs];         // rows appended by this call
+  int tok_off[kMaxSeqs + 1];   // prefix sums of n_new
+  int work_off[kMaxSeqs + 1];  // prefix sums of per-sequence work items of the attention kernel
+};
+
+struct Shape {
+  int H, KV, g, hd;
+  int cap;               // positions per (sequence, kv head)
+  long long seq_stride;  // floats between two sequences' caches = KV*cap*hd
+};
+
+struct PrepArgs {
+  const float *q, *k, *v;           // [tokens, H*hd], [tokens, KV*hd] x2: projection outputs
+  const float *b_q, *b_k, *b_v;     // nullable
+  const float *q_norm, *k_norm;     // nullable, [hd]
+  double eps;
+  const float2 *rope_tab;           // [positions][hd/2] (cos, sin)
+  float *q_rot;                     // [tokens, H*hd]
+  float *kc, *vc;
+};
+
+// bias -> QK-norm -> RoPE -> append (K rotated, V as is); rotated Q to q_rot.
+hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, int total_tokens,
+                       hipStream_t stream);
+
+// Which attention kernel a call uses.
+enum class Path { kDecodeSplitK, kPrefillMfma, kGeneric };
+Path choose_path(const SeqTable &st, const Shape &sh);
+
+// Fills st.work_off for the chosen path and returns the number of work items.
+// decode_chunk is the number of keys one decode workgroup covers (multiple of 64).
+int plan_work(SeqTable &st, const Shape &sh, Path path, int decode_chunk);
+int choose_decode_chunk(const SeqTable &st, const Shape &sh);
+
+// Floats needed for split-K partials of a decode call with `items` work items.
+size_t decode_partial_floats(const Shape &sh, int items);
+
+hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
+                         const SeqTable &st, const Shape &sh, int items, int decode_chunk, float scale,
+                         hipStream_t stream);
+hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
+                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream);
+hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
+                          const SeqTable &st, const Shape &sh, int total_tokens, float scale,
+                          hipStream_t stream);
+
+hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
+                                int num_kv_heads, int head_dim, int capacity, hipStream_t stream);
+
+}  // namespace shainet

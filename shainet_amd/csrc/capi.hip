@@ -1,0 +1,533 @@
+// C ABI of libshainet_hip_kernels.so (declared in include/shainet_hip_attn.h).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "../../include/shainet_hip_attn.h"
+#include "attn_kernels.hpp"
+
+using namespace shainet;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  return fail(e == hipErrorOutOfMemory ? SHAINET_HIP_ERR_ALLOC : SHAINET_HIP_ERR_RUNTIME, "%s: %s", what,
+              hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                  \
+  do {                                                 \
+    hipError_t e_ = (expr);                            \
+    if (e_ != hipSuccess) return hip_fail(e_, #expr);  \
+  } while (0)
+
+// Grow-only device buffer.
+struct DevBuf {
+  float *p = nullptr;
+  size_t cap = 0;  // floats
+  int reserve(size_t n) {
+    if (n <= cap) return SHAINET_HIP_OK;
+    size_t want = cap ? cap : 1024;
+    while (want < n) want *= 2;
+    float *np = nullptr;
+    hipError_t e = hipMalloc((void **)&np, want * sizeof(float));
+    if (e != hipSuccess) {  // try the exact size before giving up
+      want = n;
+      e = hipMalloc((void **)&np, want * sizeof(float));
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    if (p) (void)hipFree(p);
+    p = np;
+    cap = want;
+    return SHAINET_HIP_OK;
+  }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    cap = 0;
+  }
+};
+
+}  // namespace
+
+struct shainet_attn_ctx {
+  int H, KV, g, hd;
+  double eps;
+  float scale;  // (float)(1.0 / sqrt((double)hd)), llama_block.cr:249
+  std::vector<float> inv_freq;
+  float *d_q_norm = nullptr, *d_k_norm = nullptr;
+  float *d_bq = nullptr, *d_bk = nullptr, *d_bv = nullptr;
+  float2 *d_rope = nullptr;
+  int rope_positions = 0;
+  hipStream_t stream = nullptr;      // where work is issued
+  hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
+  DevBuf q_rot, partials, in_q, in_k, in_v, out;
+  int last_rows = 0;
+  int decode_chunk_override = 0;
+};
+
+struct shainet_kv_cache {
+  shainet_attn_ctx *ctx;
+  int batch, cap;
+  float *k = nullptr, *v = nullptr;
+  std::vector<int> len;
+};
+
+namespace {
+
+int upload(float **dst, const float *src, size_t n) {
+  if (*dst) (void)hipFree(*dst);
+  *dst = nullptr;
+  if (!src) return SHAINET_HIP_OK;
+  HIP_TRY(hipMalloc((void **)dst, (n ? n : 1) * sizeof(float)));
+  HIP_TRY(hipMemcpy(*dst, src, n * sizeof(float), hipMemcpyHostToDevice));
+  return SHAINET_HIP_OK;
+}
+
+// cos/sin of (float)pos * inv_freq[i], computed with the host's libm exactly as
+// llama_block.cr:274-277 does, for pos in [0, positions).
+int ensure_rope_table(shainet_attn_ctx *c, int positions) {
+  if (positions <= c->rope_positions) return SHAINET_HIP_OK;
+  int want = c->rope_positions ? c->rope_positions : 1024;
+  while (want < positions) want *= 2;
+  const int half = c->hd / 2;
+  if (half == 0) {
+    c->rope_positions = want;
+    return SHAINET_HIP_OK;
+  }
+  std::vector<float2> tab((size_t)want * half);
+  for (int pos = 0; pos < want; ++pos)
+    for (int i = 0; i < half; ++i) {
+      const float angle = (float)pos * c->inv_freq[i];
+      tab[(size_t)pos * half + i] = float2{cosf(angle), sinf(angle)};
+    }
+  float2 *np = nullptr;
+  HIP_TRY(hipMalloc((void **)&np, tab.size() * sizeof(float2)));
+  hipError_t e = hipMemcpy(np, tab.data(), tab.size() * sizeof(float2), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    (void)hipFree(np);
+    return hip_fail(e, "hipMemcpy(rope table)");
+  }
+  if (c->d_rope) {
+    // kernels already queued may still read the old table
+    (void)hipStreamSynchronize(c->stream);
+    (void)hipFree(c->d_rope);
+  }
+  c->d_rope = np;
+  c->rope_positions = want;
+  return SHAINET_HIP_OK;
+}
+
+Shape shape_of(const shainet_attn_ctx *c, int cap) {
+  Shape sh;
+  sh.H = c->H;
+  sh.KV = c->KV;
+  sh.g = c->g;
+  sh.hd = c->hd;
+  sh.cap = cap;
+  sh.seq_stride = (long long)c->KV * cap * c->hd;
+  return sh;
+}
+
+// Attention of already rotated rows over a cache: shared by the fused entry
+// point and by attention_kv_f32.
+int run_attention(shainet_attn_ctx *c, const float *q_rot, const float *kc, const float *vc, float *out,
+                  SeqTable &st, const Shape &sh, int total_tokens, float scale, hipStream_t stream) {
+  const Path path = choose_path(st, sh);
+  hipError_t e;
+  if (path == Path::kDecodeSplitK) {
+    const int chunk = c->decode_chunk_override ? c->decode_chunk_override : choose_decode_chunk(st, sh);
+    const int items = plan_work(st, sh, path, chunk);
+    int rc = c->partials.reserve(decode_partial_floats(sh, items));
+    if (rc) return rc;
+    e = launch_decode(q_rot, kc, vc, out, c->partials.p, st, sh, items, chunk, scale, stream);
+  } else if (path == Path::kPrefillMfma) {
+    const int items = plan_work(st, sh, path, 0);
+    e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream);
+  } else {
+    plan_work(st, sh, path, 0);
+    e = launch_generic(q_rot, kc, vc, out, st, sh, total_tokens, scale, stream);
+  }
+  if (e != hipSuccess) return hip_fail(e, "attention launch");
+  return SHAINET_HIP_OK;
+}
+
+// Context behind the two reference-named entry points: they carry no handle, so
+// they share one grow-only scratch set, as the reference's class-level scratch
+// does (llama_block.cr:57-68).
+shainet_attn_ctx *legacy_ctx() {
+  static shainet_attn_ctx *c = new (std::nothrow) shainet_attn_ctx();
+  return c;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *shainet_hip_last_error(void) { return g_err; }
+
+int shainet_hip_available(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return 0;
+  return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+}
+
+void kv_cache_append_f32(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
+                         int num_kv_heads, int head_dim, int capacity) {
+  hipError_t e = launch_legacy_append(staging, kc, vc, new_tokens, start_pos, num_kv_heads, head_dim, capacity,
+                                      nullptr);
+  if (e != hipSuccess) {
+    hip_fail(e, "kv_cache_append_f32");
+    fprintf(stderr, "HIP Error in kv_cache_append_f32: %s\n", hipGetErrorString(e));
+  }
+}
+
+void attention_kv_f32(const float *q, const float *kc, const float *vc, float *out, float *ws, int new_tokens,
+                      int start_pos, int num_heads, int heads_per_kv, int head_dim, int capacity, float scale) {
+  (void)ws;
+  shainet_attn_ctx *c = legacy_ctx();
+  if (!c || new_tokens < 1 || start_pos < 0 || heads_per_kv < 1 || num_heads % heads_per_kv != 0 ||
+      head_dim < 1 || head_dim > 256 || start_pos + new_tokens > capacity) {
+    fail(SHAINET_HIP_ERR_ARGUMENT, "attention_kv_f32: invalid arguments");
+    fprintf(stderr, "HIP Error in attention_kv_f32: invalid arguments\n");
+    return;
+  }
+  c->H = num_heads;
+  c->KV = num_heads / heads_per_kv;
+  c->g = heads_per_kv;
+  c->hd = head_dim;
+  SeqTable st;
+  memset(&st, 0, sizeof st);
+  st.n_seqs = 1;
+  st.start_pos[0] = start_pos;
+  st.n_new[0] = new_tokens;
+  st.tok_off[1] = new_tokens;
+  Shape sh = shape_of(c, capacity);
+  int rc = run_attention(c, q, kc, vc, out, st, sh, new_tokens, scale, nullptr);
+  if (rc) fprintf(stderr, "HIP Error in attention_kv_f32: %s\n", g_err);
+}
+
+int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads, int head_dim,
+                        double rope_theta, const float *rope_freqs, const float *q_norm, int q_norm_len,
+                        const float *k_norm, int k_norm_len, double qk_norm_eps, int max_positions) {
+  if (!out) return fail(SHAINET_HIP_ERR_ARGUMENT, "out is null");
+  *out = nullptr;
+  if (!(num_kv_heads > 0 && num_heads > 0 && num_heads % num_kv_heads == 0))
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "num_heads must be divisible by num_kv_heads");
+  if (head_dim <= 0) return fail(SHAINET_HIP_ERR_ARGUMENT, "head_dim must be positive");
+  if (head_dim > 256) return fail(SHAINET_HIP_ERR_ARGUMENT, "head_dim above 256 is not supported");
+  if (q_norm && q_norm_len != head_dim)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "qk_norm weight size %d != head_dim %d", q_norm_len, head_dim);
+  if (k_norm && k_norm_len != head_dim)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "qk_norm weight size %d != head_dim %d", k_norm_len, head_dim);
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  shainet_attn_ctx *c = new (std::nothrow) shainet_attn_ctx();
+  if (!c) return fail(SHAINET_HIP_ERR_ALLOC, "out of host memory");
+  c->H = num_heads;
+  c->KV = num_kv_heads;
+  c->g = num_heads / num_kv_heads;
+  c->hd = head_dim;
+  c->eps = qk_norm_eps;
+  c->scale = (float)(1.0 / sqrt((double)head_dim));
+  c->inv_freq.resize(head_dim / 2);
+  for (int i = 0; i < head_dim / 2; ++i)  // llama_block.cr:669-675
+    c->inv_freq[i] = rope_freqs ? rope_freqs[i] : (float)(1.0 / pow(rope_theta, 2.0 * i / head_dim));
+  if (const char *env = getenv("SHAINET_HIP_DECODE_CHUNK")) {
+    int v = atoi(env);
+    if (v >= 64 && v % 64 == 0) c->decode_chunk_override = v;
+  }
+  int rc = SHAINET_HIP_OK;
+  hipError_t e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
+  if (e != hipSuccess) rc = hip_fail(e, "hipStreamCreate");
+  c->stream = c->own_stream;
+  if (!rc) rc = upload(&c->d_q_norm, q_norm, head_dim);
+  if (!rc) rc = upload(&c->d_k_norm, k_norm, head_dim);
+  if (!rc) rc = ensure_rope_table(c, max_positions > 0 ? max_positions : 1024);
+  if (rc) {
+    shainet_attn_destroy(c);
+    return rc;
+  }
+  *out = c;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_set_bias(shainet_attn_ctx *c, const float *b_q, int b_q_len, const float *b_k, int b_k_len,
+                          const float *b_v, int b_v_len) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
+  const int q_dim = c->H * c->hd, kv_dim = c->KV * c->hd;
+  if (b_q && b_q_len != q_dim)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "bias size %d does not match matrix cols %d", b_q_len, q_dim);
+  if (b_k && b_k_len != kv_dim)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "bias size %d does not match matrix cols %d", b_k_len, kv_dim);
+  if (b_v && b_v_len != kv_dim)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "bias size %d does not match matrix cols %d", b_v_len, kv_dim);
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  int rc = upload(&c->d_bq, b_q, q_dim);
+  if (!rc) rc = upload(&c->d_bk, b_k, kv_dim);
+  if (!rc) rc = upload(&c->d_bv, b_v, kv_dim);
+  return rc;
+}
+
+int shainet_attn_destroy(shainet_attn_ctx *c) {
+  if (!c) return SHAINET_HIP_OK;
+  (void)hipStreamSynchronize(c->stream);
+  if (c->own_stream) {
+    (void)hipStreamSynchronize(c->own_stream);
+    (void)hipStreamDestroy(c->own_stream);
+  }
+  for (float *p : {c->d_q_norm, c->d_k_norm, c->d_bq, c->d_bk, c->d_bv})
+    if (p) (void)hipFree(p);
+  if (c->d_rope) (void)hipFree(c->d_rope);
+  for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
+  delete c;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_sync(shainet_attn_ctx *c) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  return SHAINET_HIP_OK;
+}
+
+void *shainet_attn_stream(shainet_attn_ctx *c) { return c ? (void *)c->stream : nullptr; }
+
+int shainet_attn_set_stream(shainet_attn_ctx *c, void *stream) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
+  HIP_TRY(hipStreamSynchronize(c->stream));  // nothing of ours may still run on the old one
+  c->stream = (hipStream_t)stream;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_inv_freq(shainet_attn_ctx *c, float *out) {
+  if (!c || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  memcpy(out, c->inv_freq.data(), c->inv_freq.size() * sizeof(float));
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_create(shainet_kv_cache **out, shainet_attn_ctx *ctx, int batch, int capacity) {
+  if (!out) return fail(SHAINET_HIP_ERR_ARGUMENT, "out is null");
+  *out = nullptr;
+  if (!ctx || batch < 1 || capacity < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid cache geometry");
+  shainet_kv_cache *kc = new (std::nothrow) shainet_kv_cache();
+  if (!kc) return fail(SHAINET_HIP_ERR_ALLOC, "out of host memory");
+  kc->ctx = ctx;
+  kc->batch = batch;
+  kc->cap = capacity;
+  kc->len.assign(batch, 0);
+  const size_t bytes = (size_t)batch * ctx->KV * capacity * ctx->hd * sizeof(float);
+  hipError_t e = hipMalloc((void **)&kc->k, bytes);
+  if (e == hipSuccess) e = hipMalloc((void **)&kc->v, bytes);
+  // zero-fill: rows never appended must hold finite values
+  if (e == hipSuccess) e = hipMemset(kc->k, 0, bytes);
+  if (e == hipSuccess) e = hipMemset(kc->v, 0, bytes);
+  if (e != hipSuccess) {
+    int rc = hip_fail(e, "kv cache allocation");
+    shainet_kv_cache_destroy(kc);
+    return rc;
+  }
+  *out = kc;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_destroy(shainet_kv_cache *kc) {
+  if (!kc) return SHAINET_HIP_OK;
+  if (kc->ctx) (void)hipStreamSynchronize(kc->ctx->stream);
+  if (kc->k) (void)hipFree(kc->k);
+  if (kc->v) (void)hipFree(kc->v);
+  delete kc;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_clear(shainet_kv_cache *kc, int seq) {
+  if (!kc || seq >= kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid sequence");
+  if (seq < 0)
+    kc->len.assign(kc->batch, 0);
+  else
+    kc->len[seq] = 0;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_len(const shainet_kv_cache *kc, int seq) {
+  if (!kc || seq < 0 || seq >= kc->batch) return -1;
+  return kc->len[seq];
+}
+
+int shainet_kv_cache_capacity(const shainet_kv_cache *kc) { return kc ? kc->cap : -1; }
+
+float *shainet_kv_cache_k(shainet_kv_cache *kc) { return kc ? kc->k : nullptr; }
+float *shainet_kv_cache_v(shainet_kv_cache *kc) { return kc ? kc->v : nullptr; }
+
+int shainet_kv_cache_reserve(shainet_kv_cache *kc, int capacity) {
+  if (!kc) return fail(SHAINET_HIP_ERR_ARGUMENT, "cache is null");
+  if (capacity <= kc->cap) return SHAINET_HIP_OK;
+  shainet_attn_ctx *c = kc->ctx;
+  const size_t row = (size_t)c->hd * sizeof(float);
+  const size_t bytes = (size_t)kc->batch * c->KV * capacity * row;
+  float *nk = nullptr, *nv = nullptr;
+  hipError_t e = hipMalloc((void **)&nk, bytes);
+  if (e == hipSuccess) e = hipMalloc((void **)&nv, bytes);
+  if (e == hipSuccess) e = hipMemsetAsync(nk, 0, bytes, c->stream);
+  if (e == hipSuccess) e = hipMemsetAsync(nv, 0, bytes, c->stream);
+  // one strided copy per tensor: [batch*KV] runs of cap rows into runs of capacity rows
+  if (e == hipSuccess)
+    e = hipMemcpy2DAsync(nk, (size_t)capacity * row, kc->k, (size_t)kc->cap * row, (size_t)kc->cap * row,
+                         (size_t)kc->batch * c->KV, hipMemcpyDeviceToDevice, c->stream);
+  if (e == hipSuccess)
+    e = hipMemcpy2DAsync(nv, (size_t)capacity * row, kc->v, (size_t)kc->cap * row, (size_t)kc->cap * row,
+                         (size_t)kc->batch * c->KV, hipMemcpyDeviceToDevice, c->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+  if (e != hipSuccess) {
+    if (nk) (void)hipFree(nk);
+    if (nv) (void)hipFree(nv);
+    return hip_fail(e, "kv cache growth");
+  }
+  (void)hipFree(kc->k);
+  (void)hipFree(kc->v);
+  kc->k = nk;
+  kc->v = nv;
+  kc->cap = capacity;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_fill(shainet_kv_cache *kc, int seq, const float *k_rows, const float *v_rows, int n, int mem) {
+  if (!kc || seq < 0 || seq >= kc->batch || n < 0 || !k_rows || !v_rows)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid fill arguments");
+  if (n > kc->cap) return fail(SHAINET_HIP_ERR_CAPACITY, "fill of %d rows exceeds capacity %d", n, kc->cap);
+  shainet_attn_ctx *c = kc->ctx;
+  const size_t row = (size_t)c->hd * sizeof(float);
+  const hipMemcpyKind kind = mem == SHAINET_HIP_MEM_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
+  if (n > 0) {
+    float *dk = kc->k + (size_t)seq * c->KV * kc->cap * c->hd;
+    float *dv = kc->v + (size_t)seq * c->KV * kc->cap * c->hd;
+    HIP_TRY(hipMemcpy2DAsync(dk, (size_t)kc->cap * row, k_rows, (size_t)n * row, (size_t)n * row, c->KV, kind,
+                             c->stream));
+    HIP_TRY(hipMemcpy2DAsync(dv, (size_t)kc->cap * row, v_rows, (size_t)n * row, (size_t)n * row, c->KV, kind,
+                             c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+  }
+  kc->len[seq] = n;
+  return ensure_rope_table(c, n + 1);
+}
+
+int shainet_kv_cache_read(shainet_kv_cache *kc, int seq, int kv_head, int pos0, int n, float *k_out, float *v_out) {
+  if (!kc || seq < 0 || seq >= kc->batch || kv_head < 0 || kv_head >= kc->ctx->KV || pos0 < 0 || n < 0 ||
+      pos0 + n > kc->cap)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid read arguments");
+  shainet_attn_ctx *c = kc->ctx;
+  const size_t off = (((size_t)seq * c->KV + kv_head) * kc->cap + pos0) * c->hd;
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  if (k_out && n) HIP_TRY(hipMemcpy(k_out, kc->k + off, (size_t)n * c->hd * sizeof(float), hipMemcpyDeviceToHost));
+  if (v_out && n) HIP_TRY(hipMemcpy(v_out, kc->v + off, (size_t)n * c->hd * sizeof(float), hipMemcpyDeviceToHost));
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, const int *new_tokens,
+                         int n_seqs, const float *q, const float *k, const float *v, float *out, int mem) {
+  if (!c || !kc || kc->ctx != c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (!new_tokens || !q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (n_seqs < 1 || n_seqs > SHAINET_HIP_MAX_BATCH)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", SHAINET_HIP_MAX_BATCH);
+  SeqTable st;
+  memset(&st, 0, sizeof st);
+  st.n_seqs = n_seqs;
+  long long total = 0;
+  int max_pos = 0;
+  for (int s = 0; s < n_seqs; ++s) {
+    const int slot = seq_ids ? seq_ids[s] : s;
+    if (slot < 0 || slot >= kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "sequence id %d out of range", slot);
+    for (int t = 0; t < s; ++t)
+      if (st.slot[t] == slot) return fail(SHAINET_HIP_ERR_ARGUMENT, "sequence id %d appears twice", slot);
+    if (new_tokens[s] < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "new_tokens must be positive");
+    if ((long long)kc->len[slot] + new_tokens[s] > kc->cap)
+      return fail(SHAINET_HIP_ERR_CAPACITY, "sequence %d: %d cached + %d new rows exceed capacity %d", slot,
+                  kc->len[slot], new_tokens[s], kc->cap);
+    st.slot[s] = slot;
+    st.start_pos[s] = kc->len[slot];
+    st.n_new[s] = new_tokens[s];
+    st.tok_off[s] = (int)total;
+    total += new_tokens[s];
+    if (total > 0x3fffffff) return fail(SHAINET_HIP_ERR_ARGUMENT, "too many rows in one call");
+    max_pos = max_pos > kc->len[slot] + new_tokens[s] ? max_pos : kc->len[slot] + new_tokens[s];
+  }
+  st.tok_off[n_seqs] = (int)total;
+  const int rows = (int)total;
+  const size_t q_floats = (size_t)rows * c->H * c->hd, kv_floats = (size_t)rows * c->KV * c->hd;
+  int rc = ensure_rope_table(c, max_pos);
+  if (!rc) rc = c->q_rot.reserve(q_floats);
+  if (rc) return rc;
+
+  const float *dq = q, *dk = k, *dv = v;
+  float *dout = out;
+  if (mem == SHAINET_HIP_MEM_HOST) {
+    if ((rc = c->in_q.reserve(q_floats)) || (rc = c->in_k.reserve(kv_floats)) ||
+        (rc = c->in_v.reserve(kv_floats)) || (rc = c->out.reserve(q_floats)))
+      return rc;
+    HIP_TRY(hipMemcpyAsync(c->in_q.p, q, q_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(hipMemcpyAsync(c->in_k.p, k, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(hipMemcpyAsync(c->in_v.p, v, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    dq = c->in_q.p;
+    dk = c->in_k.p;
+    dv = c->in_v.p;
+    dout = c->out.p;
+  } else if (mem != SHAINET_HIP_MEM_DEVICE) {
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "mem must be SHAINET_HIP_MEM_HOST or SHAINET_HIP_MEM_DEVICE");
+  }
+
+  Shape sh = shape_of(c, kc->cap);
+  PrepArgs pa;
+  pa.q = dq;
+  pa.k = dk;
+  pa.v = dv;
+  pa.b_q = c->d_bq;
+  pa.b_k = c->d_bk;
+  pa.b_v = c->d_bv;
+  pa.q_norm = c->d_q_norm;
+  pa.k_norm = c->d_k_norm;
+  pa.eps = c->eps;
+  pa.rope_tab = c->d_rope;
+  pa.q_rot = c->q_rot.p;
+  pa.kc = kc->k;
+  pa.vc = kc->v;
+  hipError_t e = launch_prep(pa, st, sh, rows, c->stream);
+  if (e != hipSuccess) return hip_fail(e, "prep launch");
+  // the rows are in the cache from here on: @cache_len = total_len (llama_block.cr:288-289)
+  for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
+  c->last_rows = rows;
+  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream);
+  if (rc) return rc;
+  if (mem == SHAINET_HIP_MEM_HOST) {
+    HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+  }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_last_q_rot(shainet_attn_ctx *c, float *out, int rows) {
+  if (!c || !out || rows < 0 || rows > c->last_rows) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  HIP_TRY(hipMemcpy(out, c->q_rot.p, (size_t)rows * c->H * c->hd * sizeof(float), hipMemcpyDeviceToHost));
+  return SHAINET_HIP_OK;
+}
+
+}  // extern "C"

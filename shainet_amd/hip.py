@@ -1,0 +1,293 @@
+"""ctypes binding of libshainet_hip_kernels.so.
+
+`HIP` plays the role SHAInet::CUDA plays in the reference for this path
+(src/shainet/cuda.cr:778-891): availability probes and the two kernel entry
+points with the reference's names; `AttnContext` / `KVCache` wrap the fused
+batched entry points.  There is no CPU fallback: a missing library or a missing
+GPU raises.
+"""
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.join(_HERE, "csrc")
+_SO = os.path.join(_HERE, "lib", "libshainet_hip_kernels.so")
+
+MEM_HOST, MEM_DEVICE = 0, 1
+MAX_BATCH = 64
+
+_f32p = C.POINTER(C.c_float)
+_i32p = C.POINTER(C.c_int)
+
+
+class HipError(RuntimeError):
+    pass
+
+
+class ArgumentError(ValueError):
+    """What the Crystal layer raises as ArgumentError."""
+
+
+def library_path():
+    return _SO
+
+
+def build_library(force=True):
+    """Compile the HIP library for gfx950 (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", _CSRC, "-j8"] + (["-B"] if force else [])
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise HipError("building libshainet_hip_kernels.so failed:\n" + proc.stdout[-4000:])
+    return _SO
+
+
+_lib = None
+
+_SIGNATURES = {
+    "shainet_hip_last_error": (C.c_char_p, []),
+    "shainet_hip_available": (C.c_int, []),
+    "kv_cache_append_f32": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "attention_kv_f32": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "shainet_attn_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_double, _f32p, _f32p,
+                                      C.c_int, _f32p, C.c_int, C.c_double, C.c_int]),
+    "shainet_attn_set_bias": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p, C.c_int, _f32p, C.c_int]),
+    "shainet_attn_destroy": (C.c_int, [C.c_void_p]),
+    "shainet_attn_sync": (C.c_int, [C.c_void_p]),
+    "shainet_attn_stream": (C.c_void_p, [C.c_void_p]),
+    "shainet_attn_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "shainet_attn_inv_freq": (C.c_int, [C.c_void_p, _f32p]),
+    "shainet_kv_cache_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_int]),
+    "shainet_kv_cache_destroy": (C.c_int, [C.c_void_p]),
+    "shainet_kv_cache_clear": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_kv_cache_len": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_kv_cache_capacity": (C.c_int, [C.c_void_p]),
+    "shainet_kv_cache_reserve": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_kv_cache_k": (C.c_void_p, [C.c_void_p]),
+    "shainet_kv_cache_v": (C.c_void_p, [C.c_void_p]),
+    "shainet_kv_cache_fill": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
+    "shainet_kv_cache_read": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p]),
+    "shainet_attn_forward": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.c_void_p, C.c_int]),
+    "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
+}
+
+
+def exported_symbols():
+    """Every symbol include/shainet_hip_attn.h declares."""
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise HipError(f"{_SO} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                           "(there is no CPU fallback)")
+        L = C.CDLL(_SO)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc == 0:
+        return
+    msg = lib().shainet_hip_last_error().decode()
+    if rc == 1:
+        raise ArgumentError(msg)
+    raise HipError(f"status {rc}: {msg}")
+
+
+def _ptr(x):
+    """Device or host address of a torch tensor / numpy array / int."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    return x.ctypes.data
+
+
+def _f32_arr(a):
+    import numpy as np
+
+    if a is None:
+        return None, None, -1
+    arr = np.ascontiguousarray(a, dtype=np.float32)
+    return arr, arr.ctypes.data_as(_f32p), arr.size
+
+
+class HIP:
+    """Counterpart of SHAInet::CUDA for the attention path."""
+
+    @staticmethod
+    def kernels_available():
+        # cuda.cr:111-122: can the kernel library be opened?
+        try:
+            lib()
+            return True
+        except (HipError, OSError):
+            return False
+
+    @staticmethod
+    def available():
+        if os.environ.get("SHAINET_DISABLE_HIP"):  # cuda.cr:64 (SHAINET_DISABLE_CUDA)
+            return False
+        return HIP.kernels_available() and bool(lib().shainet_hip_available())
+
+    @staticmethod
+    def fully_available():
+        return HIP.available() and HIP.kernels_available()  # cuda.cr:778-780
+
+    @staticmethod
+    def kv_cache_append_f32(staging, kc, vc, new_tokens, start_pos, num_kv_heads, head_dim, capacity):
+        lib().kv_cache_append_f32(_ptr(staging), _ptr(kc), _ptr(vc), new_tokens, start_pos, num_kv_heads, head_dim,
+                                  capacity)
+
+    @staticmethod
+    def attention_kv_f32(q, kc, vc, out, ws, new_tokens, start_pos, num_heads, heads_per_kv, head_dim, capacity,
+                         scale):
+        lib().attention_kv_f32(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), _ptr(ws), new_tokens, start_pos, num_heads,
+                               heads_per_kv, head_dim, capacity, scale)
+
+
+class AttnContext:
+    """Attention parameters of one LlamaBlock (llama_block.cr:10-28, 73-108)."""
+
+    def __init__(self, num_heads, num_kv_heads, head_dim, rope_theta=10000.0, rope_freqs=None, q_norm=None,
+                 k_norm=None, eps=1e-6, max_positions=1024):
+        self._h = C.c_void_p()
+        _, fp, _ = self._keep_f = _f32_arr(rope_freqs)
+        _, qp, qn = self._keep_q = _f32_arr(q_norm)
+        _, kp, kn = self._keep_k = _f32_arr(k_norm)
+        _check(lib().shainet_attn_create(C.byref(self._h), num_heads, num_kv_heads, head_dim, rope_theta, fp, qp, qn,
+                                         kp, kn, eps, max_positions))
+        self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
+        self.q_dim, self.kv_dim = num_heads * head_dim, num_kv_heads * head_dim
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().shainet_attn_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def set_bias(self, b_q, b_k, b_v):
+        a = [_f32_arr(b) for b in (b_q, b_k, b_v)]
+        _check(lib().shainet_attn_set_bias(self._h, a[0][1], a[0][2], a[1][1], a[1][2], a[2][1], a[2][2]))
+
+    def sync(self):
+        _check(lib().shainet_attn_sync(self._h))
+
+    @property
+    def stream(self):
+        return lib().shainet_attn_stream(self._h)
+
+    def set_stream(self, stream_ptr):
+        _check(lib().shainet_attn_set_stream(self._h, stream_ptr))
+
+    def inv_freq(self):
+        import numpy as np
+
+        out = np.empty(self.head_dim // 2, np.float32)
+        _check(lib().shainet_attn_inv_freq(self._h, out.ctypes.data_as(_f32p)))
+        return out
+
+    def last_q_rot(self, rows):
+        import numpy as np
+
+        out = np.empty((rows, self.q_dim), np.float32)
+        _check(lib().shainet_attn_last_q_rot(self._h, out.ctypes.data_as(_f32p), rows))
+        return out
+
+    def forward(self, cache, q, k, v, new_tokens, seq_ids=None, out=None):
+        """llama_block.cr:256-296 for len(new_tokens) sequences.  numpy inputs run the
+        synchronous host-pointer mode and return numpy; torch CUDA tensors run the
+        asynchronous device-pointer mode on the context's stream."""
+        import numpy as np
+
+        n = len(new_tokens)
+        nt = (C.c_int * n)(*new_tokens)
+        ids = (C.c_int * n)(*seq_ids) if seq_ids is not None else None
+        rows = sum(new_tokens)
+        if isinstance(q, np.ndarray):
+            q, k, v = (np.ascontiguousarray(a, np.float32) for a in (q, k, v))
+            assert q.shape == (rows, self.q_dim) and k.shape == (rows, self.kv_dim) and v.shape == k.shape
+            out = np.empty((rows, self.q_dim), np.float32)
+            mem = MEM_HOST
+        else:
+            assert q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+            assert tuple(q.shape) == (rows, self.q_dim) and tuple(k.shape) == (rows, self.kv_dim)
+            if out is None:
+                import torch
+
+                out = torch.empty_like(q)
+            mem = MEM_DEVICE
+        _check(lib().shainet_attn_forward(self._h, cache._h, ids, nt, n, _ptr(q), _ptr(k), _ptr(v), _ptr(out), mem))
+        return out
+
+
+class KVCache:
+    """Device-resident fp32 KV cache: [batch][num_kv_heads][capacity][head_dim] for K and V."""
+
+    def __init__(self, ctx, batch, capacity):
+        self.ctx = ctx
+        self._h = C.c_void_p()
+        _check(lib().shainet_kv_cache_create(C.byref(self._h), ctx._h, batch, capacity))
+        self.batch = batch
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            lib().shainet_kv_cache_destroy(self._h)
+        self._h = None
+
+    __del__ = close
+
+    def clear(self, seq=-1):
+        _check(lib().shainet_kv_cache_clear(self._h, seq))
+
+    def len(self, seq=0):
+        return lib().shainet_kv_cache_len(self._h, seq)
+
+    @property
+    def capacity(self):
+        return lib().shainet_kv_cache_capacity(self._h)
+
+    def reserve(self, capacity):
+        _check(lib().shainet_kv_cache_reserve(self._h, capacity))
+
+    @property
+    def k_ptr(self):
+        return lib().shainet_kv_cache_k(self._h)
+
+    @property
+    def v_ptr(self):
+        return lib().shainet_kv_cache_v(self._h)
+
+    def fill(self, seq, k_rows, v_rows):
+        """k_rows, v_rows: [num_kv_heads, n, head_dim], K already rotated."""
+        import numpy as np
+
+        if isinstance(k_rows, np.ndarray):
+            k_rows, v_rows = (np.ascontiguousarray(a, np.float32) for a in (k_rows, v_rows))
+            mem = MEM_HOST
+        else:
+            assert k_rows.is_cuda and k_rows.is_contiguous() and v_rows.is_contiguous()
+            mem = MEM_DEVICE
+        assert tuple(k_rows.shape) == tuple(v_rows.shape) and k_rows.shape[0] == self.ctx.num_kv_heads
+        assert k_rows.shape[2] == self.ctx.head_dim
+        _check(lib().shainet_kv_cache_fill(self._h, seq, _ptr(k_rows), _ptr(v_rows), k_rows.shape[1], mem))
+
+    def read(self, seq, kv_head, pos0, n):
+        import numpy as np
+
+        k = np.empty((n, self.ctx.head_dim), np.float32)
+        v = np.empty((n, self.ctx.head_dim), np.float32)
+        _check(lib().shainet_kv_cache_read(self._h, seq, kv_head, pos0, n, k.ctypes.data_as(_f32p),
+                                           v.ctypes.data_as(_f32p)))
+        return k, v

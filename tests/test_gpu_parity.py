@@ -1,0 +1,396 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real MI355X.
+
+Bar (fp32): |gpu - oracle| <= 1e-4 + 1e-3*|oracle| elementwise; rotated Q rows and
+cache contents (RoPE positions, cache indexing) bit-identical.
+"""
+import numpy as np
+import pytest
+
+import refmath as rm
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import shainet_amd as sa
+
+    assert sa.HIP.fully_available(), "no gfx950 device or libshainet_hip_kernels.so missing"
+    return sa
+
+
+def make_pair(hip, H, KV, hd, theta=10000.0, norm=False, bias=False, freqs=None, batch=1, capacity=512, seed=0,
+              eps=1e-6):
+    r = np.random.default_rng(seed)
+    qn = kn = None
+    if norm:
+        qn = (1 + 0.02 * r.standard_normal(hd)).astype(np.float32)
+        kn = (1 + 0.02 * r.standard_normal(hd)).astype(np.float32)
+    ctx = hip.AttnContext(H, KV, hd, rope_theta=theta, rope_freqs=freqs, q_norm=qn, k_norm=kn, eps=eps)
+    cache = hip.KVCache(ctx, batch, capacity)
+    blocks = []
+    for _ in range(batch):
+        b = orc.Block(H * hd, H, KV, hd, eps=eps, rope_theta=theta)
+        if freqs is not None:
+            b.set_rope(theta, freqs)
+        if norm:
+            b.set_qk_norm(qn, kn)
+        blocks.append(b)
+    if bias:
+        bq, bk, bv = (0.3 * r.standard_normal(n * hd).astype(np.float32) for n in (H, KV, KV))
+        ctx.set_bias(bq, bk, bv)
+        for b in blocks:
+            b.set_bias(bq, bk, bv)
+    return ctx, cache, blocks, r
+
+
+def rows(r, T, H, KV, hd):
+    return tuple(r.standard_normal((T, n * hd)).astype(np.float32) for n in (H, KV, KV))
+
+
+def check_step(ctx, cache, blocks, r, new_tokens, seq_ids=None, threads=8, what=""):
+    """One forward call on both sides; returns the max abs error."""
+    H, KV, hd = ctx.num_heads, ctx.num_kv_heads, ctx.head_dim
+    ids = list(range(len(new_tokens))) if seq_ids is None else seq_ids
+    parts = [rows(r, T, H, KV, hd) for T in new_tokens]
+    q, k, v = (np.concatenate([p[i] for p in parts]) for i in range(3))
+    got = ctx.forward(cache, q, k, v, new_tokens, seq_ids)
+    want = np.concatenate([blocks[s].attention_cached_qkv(*p, threads=threads) for s, p in zip(ids, parts)])
+    err = rm.assert_close(got, want, ATOL, RTOL, what)
+    for s in ids:
+        assert cache.len(s) == blocks[s].cache_len
+    return err
+
+
+def check_cache_bits(cache, blocks, seqs=None):
+    for s in (range(len(blocks)) if seqs is None else seqs):
+        n = blocks[s].cache_len
+        for c in range(blocks[s].num_kv_heads):
+            k, v = cache.read(s, c, 0, n)
+            assert np.array_equal(k.view(np.uint32), blocks[s].k_cache(c).view(np.uint32)), "K cache bits differ"
+            assert np.array_equal(v.view(np.uint32), blocks[s].v_cache(c).view(np.uint32)), "V cache bits differ"
+
+
+# ------------------------------------------------------------------ the reference's own scenarios
+def test_reference_gqa_prefill_then_decode(hip):
+    # spec/llama_attention_gpu_spec.cr:16-66: d=64, 8 heads, 4 kv heads (g=2), prefill 6 + 3 decodes
+    ctx, cache, blocks, r = make_pair(hip, 8, 4, 8, seed=42)
+    for T in (6, 1, 1, 1):
+        check_step(ctx, cache, blocks, r, [T])
+    check_cache_bits(cache, blocks)
+
+
+def test_reference_growth_and_clear(hip):
+    # spec/llama_attention_gpu_spec.cr:68-104: d=32, 4 heads, 2 kv heads, 290 + 10 rows across the
+    # initial capacity 256; a rerun after clear must give the same results (no stale rows leak)
+    ctx, cache, blocks, r0 = make_pair(hip, 4, 2, 8, seed=7, capacity=256)
+    H, KV, hd = 4, 2, 8
+    steps = [rows(r0, T, H, KV, hd) for T in [200, 56] + [1] * 4]
+    grow_at = 2
+    outs = []
+    for run in range(2):
+        cache.clear()
+        blocks[0].clear_cache()
+        res = []
+        for i, p in enumerate(steps + [rows(np.random.default_rng(99), 34, H, KV, hd)]):
+            if cache.len(0) + p[0].shape[0] > cache.capacity:
+                with pytest.raises(hip.HipError):
+                    ctx.forward(cache, *p, [p[0].shape[0]])
+                assert i >= grow_at
+                cache.reserve(2 * cache.capacity)
+            got = ctx.forward(cache, *p, [p[0].shape[0]])
+            want = blocks[0].attention_cached_qkv(*p)
+            rm.assert_close(got, want, ATOL, RTOL, f"run {run} step {i}")
+            res.append(got)
+        outs.append(res)
+        assert cache.len(0) == 294 and cache.capacity == 512
+        check_cache_bits(cache, blocks)
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b)
+
+
+def test_bias_nil_equals_zero_and_size_check(hip):
+    # spec/llama_qkv_bias_spec.cr:8-72
+    H, KV, hd = 2, 2, 4
+    a = hip.AttnContext(H, KV, hd)
+    b = hip.AttnContext(H, KV, hd)
+    b.set_bias(np.zeros(8), np.zeros(8), np.zeros(8))
+    c = hip.AttnContext(H, KV, hd)
+    c.set_bias(0.3 * np.arange(1, 9), 0.2 * np.arange(1, 9), 0.5 * np.arange(1, 9))
+    q, k, v = rows(np.random.default_rng(1), 1, H, KV, hd)
+    outs = [x.forward(hip.KVCache(x, 1, 8), q, k, v, [1]) for x in (a, b, c)]
+    assert np.array_equal(outs[0], outs[1])
+    assert np.abs(outs[2] - outs[0]).sum() > 0.01
+    with pytest.raises(hip.ArgumentError):
+        a.set_bias(np.zeros(7), np.zeros(8), np.zeros(8))
+    with pytest.raises(hip.ArgumentError):
+        hip.AttnContext(8, 3, 4)
+    with pytest.raises(hip.ArgumentError):
+        hip.AttnContext(2, 2, 4, q_norm=np.ones(3), k_norm=np.ones(4))
+
+
+# ------------------------------------------------------------------ exactness of RoPE positions and cache indexing
+@pytest.mark.parametrize("H,KV,hd,theta,norm,bias", [
+    (32, 8, 64, 500000.0, False, False),
+    (32, 8, 128, 1e6, True, False),
+    (8, 2, 16, 1e6, True, True),
+    (4, 4, 7, 10000.0, False, True),  # odd head_dim: the last slot of rotated rows is 0
+])
+def test_rotated_q_and_cache_are_bit_identical(hip, H, KV, hd, theta, norm, bias):
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, theta, norm, bias, capacity=64, seed=3)
+    b = blocks[0]
+    for T in (5, 1, 9):
+        q, k, v = rows(r, T, H, KV, hd)
+        ctx.forward(cache, q, k, v, [T])
+        b.attention_cached_qkv(q, k, v, keep_q_rot=True)
+        got_q = ctx.last_q_rot(T)
+        assert np.array_equal(got_q.view(np.uint32), b.last_q_rot.view(np.uint32)), "rotated Q bits differ"
+    check_cache_bits(cache, blocks)
+    # the rotation really depends on the position: same row, two positions, different K
+    k0, _ = cache.read(0, 0, 0, 15)
+    assert k0.shape == (15, hd) and not np.array_equal(k0[1], k0[2])
+
+
+# ------------------------------------------------------------------ decode (split-K kernel)
+def test_config1_llama1b_decode_on_prefilled_cache(hip):
+    # Llama-3.2-1B head geometry, cache pre-filled to 512 positions, one new row
+    H, KV, hd, S = 32, 8, 64, 512
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, capacity=1024, seed=11)
+    kf, vf = (r.standard_normal((KV, S, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    for _ in range(3):
+        check_step(ctx, cache, blocks, r, [1])
+    check_cache_bits(cache, blocks)
+
+
+@pytest.mark.parametrize("S", [1024, 4096, 16384])
+def test_config2_decode_steps_appending(hip, S):
+    H, KV, hd = 32, 8, 64
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, capacity=S + 256, seed=S)
+    kf, vf = (r.standard_normal((KV, S, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    steps = 128 if S == 1024 else 16
+    worst = max(check_step(ctx, cache, blocks, r, [1], what=f"S={S} step {i}") for i in range(steps))
+    assert cache.len(0) == S + steps
+    assert worst < 1e-4
+
+
+def test_decode_every_length_around_tile_and_chunk_edges(hip):
+    H, KV, hd = 8, 2, 128
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, capacity=300, seed=5)
+    for i in range(270):  # lengths 1..270 cross 16-key tiles, 64-key wave strides and chunk edges
+        check_step(ctx, cache, blocks, r, [1], threads=1, what=f"len {i + 1}")
+
+
+@pytest.mark.parametrize("g,hd", [(1, 64), (2, 128), (8, 128), (16, 64)])
+def test_decode_group_sizes(hip, g, hd):
+    KV = 2
+    ctx, cache, blocks, r = make_pair(hip, KV * g, KV, hd, 1e6, capacity=1500, seed=g)
+    kf, vf = (r.standard_normal((KV, 1100, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    for _ in range(2):
+        check_step(ctx, cache, blocks, r, [1])
+
+
+def test_config3_qwen3_8b_batch16_varlen_decode(hip):
+    import torch
+
+    H, KV, hd, B = 32, 8, 128, 16
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, batch=B, capacity=8192 + 8, seed=33)
+    lens = r.integers(2048, 8193, B)
+    gen = torch.Generator(device="cuda").manual_seed(33)
+    for s in range(B):
+        kf = torch.randn((KV, int(lens[s]), hd), generator=gen, device="cuda")
+        vf = torch.randn((KV, int(lens[s]), hd), generator=gen, device="cuda")
+        torch.cuda.synchronize()
+        cache.fill(s, kf, vf)
+        blocks[s].fill_cache(kf.cpu().numpy(), vf.cpu().numpy())
+    for i in range(2):
+        err = check_step(ctx, cache, blocks, r, [1] * B, what=f"step {i}")
+        assert err < 1e-4
+    # a subset of the sequences, in another order
+    check_step(ctx, cache, blocks, r, [1] * 3, seq_ids=[7, 2, 11])
+
+
+def test_config5b_long_context_batch4_decode(hip):
+    import torch
+
+    H, KV, hd, B, S = 32, 4, 128, 4, 32768
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, batch=B, capacity=S + 8, seed=55)
+    gen = torch.Generator(device="cuda").manual_seed(55)
+    for s in range(B):
+        kf = torch.randn((KV, S, hd), generator=gen, device="cuda")
+        vf = torch.randn((KV, S, hd), generator=gen, device="cuda")
+        torch.cuda.synchronize()
+        cache.fill(s, kf, vf)
+        blocks[s].fill_cache(kf.cpu().numpy(), vf.cpu().numpy())
+    assert check_step(ctx, cache, blocks, r, [1] * B) < 1e-4
+
+
+# ------------------------------------------------------------------ prefill (MFMA kernel)
+@pytest.mark.parametrize("H,KV,hd,S,T,norm", [
+    (8, 2, 64, 0, 1, False),      # T*g < one tile
+    (8, 2, 64, 0, 33, False),
+    (8, 2, 128, 17, 70, True),    # chunked prefill on a cached prefix, partial last block
+    (6, 2, 64, 5, 45, False),     # g = 3: virtual rows straddle rows unevenly
+    (4, 4, 128, 0, 130, True),    # g = 1
+    (16, 1, 64, 40, 9, False),    # g = 16
+])
+def test_prefill_small_shapes(hip, H, KV, hd, S, T, norm):
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=norm, capacity=256, seed=T)
+    if S:
+        check_step(ctx, cache, blocks, r, [S])
+    check_step(ctx, cache, blocks, r, [T])
+    check_step(ctx, cache, blocks, r, [2])
+    check_cache_bits(cache, blocks)
+
+
+def test_prefill_then_decode_equals_one_prefill(hip):
+    # chunking invariance: T rows at once == in chunks == row by row (to fp32 round-off)
+    H, KV, hd, T = 8, 2, 64, 97
+    q, k, v = rows(np.random.default_rng(8), T, H, KV, hd)
+    outs = []
+    for chunks in ([T], [40, 57], [96, 1], [1] * T):
+        ctx = hip.AttnContext(H, KV, hd, rope_theta=500000.0)
+        cache = hip.KVCache(ctx, 1, 128)
+        o, res = 0, []
+        for n in chunks:
+            res.append(ctx.forward(cache, q[o:o + n], k[o:o + n], v[o:o + n], [n]))
+            o += n
+        outs.append(np.concatenate(res))
+    for o in outs[1:]:
+        assert np.abs(o - outs[0]).max() < 2e-5
+
+
+def test_config4_prefill_2048(hip):
+    H, KV, hd, T = 32, 8, 64, 2048
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, capacity=T + 64, seed=44)
+    assert check_step(ctx, cache, blocks, r, [T], threads=16) < 1e-4
+    check_step(ctx, cache, blocks, r, [1])
+
+
+def test_config5a_chunked_prefill_on_long_prefix_reduced(hip):
+    # Qwen3-30B-A3B geometry (32 q / 4 kv heads, hd 128, QK-norm); 512 new rows on 4096 cached
+    H, KV, hd, S, T = 32, 4, 128, 4096, 512
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, capacity=S + T, seed=51)
+    kf, vf = (r.standard_normal((KV, S, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    assert check_step(ctx, cache, blocks, r, [T], threads=16) < 1e-4
+
+
+def test_batched_prefill_mixed_lengths(hip):
+    H, KV, hd = 8, 2, 64
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, batch=4, capacity=400, seed=9)
+    check_step(ctx, cache, blocks, r, [100, 1, 37, 260])
+    check_step(ctx, cache, blocks, r, [1, 1, 1, 1])          # decode kernel, unequal lengths
+    check_step(ctx, cache, blocks, r, [5, 64], seq_ids=[2, 0])
+    check_cache_bits(cache, blocks)
+
+
+# ------------------------------------------------------------------ properties at full size
+def test_full_size_properties_prefill_8192(hip):
+    """T = 8192 (Llama-1B geometry): too slow for the scalar oracle on every row, so check
+    (a) sampled rows against the oracle run on just those rows, (b) causality, (c) GQA sharing."""
+    import torch
+
+    H, KV, hd, T = 32, 8, 64, 8192
+    ctx = hip.AttnContext(H, KV, hd, rope_theta=500000.0)
+    cache = hip.KVCache(ctx, 1, T)
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    q = torch.randn((T, H * hd), generator=gen, device="cuda")
+    k = torch.randn((T, KV * hd), generator=gen, device="cuda")
+    v = torch.randn((T, KV * hd), generator=gen, device="cuda")
+    q.view(T, KV, 4, hd)[:, :, 1] = q.view(T, KV, 4, hd)[:, :, 0]  # heads 4c and 4c+1 share a query
+    torch.cuda.synchronize()
+    out = ctx.forward(cache, q, k, v, [T])
+    ctx.sync()
+    o = out.cpu().numpy().reshape(T, H, hd)
+    assert np.isfinite(o).all()
+    assert np.array_equal(o[:, 0::4], o[:, 1::4])            # equal queries of a group -> equal outputs
+    assert np.abs(o[0] - v[0].cpu().numpy().reshape(KV, 1, hd).repeat(4, 1).reshape(H, hd)).max() < 1e-6
+    # oracle on sampled rows: fill its cache with the GPU's cache (bit-identical by the tests above)
+    b = orc.Block(H * hd, H, KV, hd, rope_theta=500000.0)
+    qh, kh, vh = q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
+    for pos in (1, 31, 32, 33, 127, 128, 4095, 4096, 8191):
+        kc = np.stack([cache.read(0, c, 0, pos)[0] for c in range(KV)])
+        vc = np.stack([cache.read(0, c, 0, pos)[1] for c in range(KV)])
+        b.fill_cache(kc, vc)
+        want = b.attention_cached_qkv(qh[pos:pos + 1], kh[pos:pos + 1], vh[pos:pos + 1], threads=8)
+        rm.assert_close(o[pos].reshape(1, -1), want, ATOL, RTOL, f"row {pos}")
+    # causality: changing rows >= 5000 leaves outputs of rows < 5000 bit-identical
+    k2, v2 = k.clone(), v.clone()
+    k2[5000:] += 1.0
+    v2[5000:] -= 1.0
+    cache.clear()
+    torch.cuda.synchronize()
+    out2 = ctx.forward(cache, q, k2, v2, [T])
+    ctx.sync()
+    assert torch.equal(out2[:5000], out[:5000]) and not torch.equal(out2[5000:], out[5000:])
+
+
+# ------------------------------------------------------------------ entry points with the reference's names
+@pytest.mark.parametrize("H,g,hd,S,T", [(8, 2, 8, 0, 6), (8, 2, 8, 6, 1), (32, 4, 64, 300, 1), (32, 4, 64, 0, 200),
+                                        (32, 8, 128, 100, 40)])
+def test_reference_named_entry_points(hip, H, g, hd, S, T):
+    import torch
+
+    KV, cap = H // g, 512
+    r = np.random.default_rng(H + S + T)
+    b = orc.Block(H * hd, H, KV, hd)
+    if S:
+        b.attention_cached_qkv(*rows(r, S, H, KV, hd))
+    q, k, v = rows(r, T, H, KV, hd)
+    kc = torch.zeros((KV, cap, hd), device="cuda")
+    vc = torch.zeros((KV, cap, hd), device="cuda")
+    for c in range(KV):
+        kc[c, :S] = torch.from_numpy(b.k_cache(c)) if S else kc[c, :S]
+        vc[c, :S] = torch.from_numpy(b.v_cache(c)) if S else vc[c, :S]
+    want = b.attention_cached_qkv(q, k, v)
+    # host side of attention_heads_gpu (llama_block.cr:432-467): staging = K tails, V tails, rotated Q
+    k_new = np.stack([b.k_cache(c)[S:] for c in range(KV)])
+    v_new = np.stack([b.v_cache(c)[S:] for c in range(KV)])
+    invf = b.inv_freq()
+    ang = (np.arange(S, S + T, dtype=np.float32)[:, None] * invf[None]).astype(np.float32)
+    cs, sn = np.cos(ang).astype(np.float32)[:, None], np.sin(ang).astype(np.float32)[:, None]
+    qh = q.reshape(T, H, hd)
+    x0, x1 = qh[..., :hd // 2], qh[..., hd // 2:]
+    q_rot = np.concatenate([x0 * cs - x1 * sn, x1 * cs + x0 * sn], -1).reshape(T, H * hd).astype(np.float32)
+    staging = torch.from_numpy(np.concatenate([k_new.ravel(), v_new.ravel(), q_rot.ravel()])).cuda()
+    out = torch.empty((T, H * hd), device="cuda")
+    torch.cuda.synchronize()
+    hip.HIP.kv_cache_append_f32(staging, kc, vc, T, S, KV, hd, cap)
+    hip.HIP.attention_kv_f32(staging[2 * k_new.size:], kc, vc, out, None, T, S, H, g, hd, cap, b.scale())
+    torch.cuda.synchronize()
+    rm.assert_close(out.cpu().numpy(), want, ATOL, RTOL)
+    assert torch.equal(kc[:, S:S + T].cpu(), torch.from_numpy(k_new))
+
+
+def test_device_pointer_mode_matches_host_pointer_mode(hip):
+    import torch
+
+    H, KV, hd = 32, 8, 128
+    r = np.random.default_rng(2)
+    parts = [rows(r, T, H, KV, hd) for T in (300, 1, 1)]
+    res = []
+    for dev in (False, True):
+        ctx = hip.AttnContext(H, KV, hd, rope_theta=1e6)
+        cache = hip.KVCache(ctx, 1, 512)
+        outs = []
+        for p in parts:
+            if dev:
+                t = [torch.from_numpy(a).cuda() for a in p]
+                torch.cuda.synchronize()
+                o = ctx.forward(cache, *t, [p[0].shape[0]])
+                ctx.sync()
+                outs.append(o.cpu().numpy())
+            else:
+                outs.append(ctx.forward(cache, *p, [p[0].shape[0]]))
+        res.append(np.concatenate(outs))
+    assert np.array_equal(res[0], res[1])
