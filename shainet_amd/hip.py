@@ -85,6 +85,13 @@ def lib():
         if not os.path.exists(_SO):
             raise HipError(f"{_SO} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
                            "(there is no CPU fallback)")
+        # A process may hold only one HIP runtime.  PyTorch ships its own copy under the
+        # same soname; when torch is installed it must be loaded first so that this
+        # library binds to that copy instead of bringing in a second one.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = C.CDLL(_SO)
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(L, name)
