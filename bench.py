@@ -1,0 +1,294 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A "step" is one layer-step of the hot path over one batch of synthetic rows:
+bias/QK-norm/RoPE/append of the new rows plus causal GQA attention over the
+device cache, through the C ABI with inputs already resident in HBM.
+
+Headline workload (BASELINE.json configs[2], the one the decode target is quoted
+on): Qwen3-8B-shaped decode, 32 Q / 8 KV heads, head_dim 128, QK-norm, theta 1e6,
+fp32, batch 16 with cached lengths drawn uniform in [2048, 8192].  The other
+configurations are timed as well and reported under "workloads".
+
+Prints ONE JSON line.  `value` is microseconds per layer-step of the headline
+workload (whole step: prep + split-K + combine kernels); `roofline` prices the
+split-K decode kernel against HBM, `roofline_prefill` the MFMA prefill kernel
+against the fp32 matrix peak; `cpu_baseline` times the CPU oracle (a C
+restatement of the reference's single-threaded Crystal path) on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def decode_bytes(KV, hd, visible):
+    """Algorithmic bytes of one decode layer-step: K and V rows read once per kv head."""
+    return sum(2 * KV * hd * 4 * L for L in visible)
+
+
+def prefill_flops(H, hd, S, T):
+    """Unmasked pairs only, 2 FLOP per MAC, QK^T and PV."""
+    return 4 * hd * H * (T * S + T * (T + 1) // 2)
+
+
+class Workload:
+    def __init__(self, sa, torch, name, H, KV, hd, theta, norm, lens, T, seed):
+        self.sa, self.torch, self.name = sa, torch, name
+        self.H, self.KV, self.hd, self.T, self.lens = H, KV, hd, T, list(lens)
+        self.B = len(self.lens)
+        self.gen = torch.Generator(device="cuda").manual_seed(seed)
+        qn = kn = None
+        if norm:
+            qn = (1 + 0.02 * torch.randn(hd, generator=self.gen, device="cuda")).cpu().numpy()
+            kn = (1 + 0.02 * torch.randn(hd, generator=self.gen, device="cuda")).cpu().numpy()
+        self.qn, self.kn, self.theta = qn, kn, theta
+        self.ctx = sa.AttnContext(H, KV, hd, rope_theta=theta, q_norm=qn, k_norm=kn, eps=1e-6,
+                                  max_positions=max(self.lens) + 4096)
+        self.cache = None
+
+    def alloc(self, extra_rows):
+        torch = self.torch
+        self.cache = self.sa.KVCache(self.ctx, self.B, max(self.lens) + extra_rows)
+        for s, L in enumerate(self.lens):
+            if L:
+                k = torch.randn((self.KV, L, self.hd), generator=self.gen, device="cuda")
+                v = torch.randn((self.KV, L, self.hd), generator=self.gen, device="cuda")
+                torch.cuda.synchronize()
+                self.cache.fill(s, k, v)
+        torch.cuda.synchronize()
+
+    def rows(self, n_steps):
+        torch = self.torch
+        R = self.B * self.T
+        q = torch.randn((n_steps, R, self.H * self.hd), generator=self.gen, device="cuda")
+        k = torch.randn((n_steps, R, self.KV * self.hd), generator=self.gen, device="cuda")
+        v = torch.randn((n_steps, R, self.KV * self.hd), generator=self.gen, device="cuda")
+        out = torch.empty((R, self.H * self.hd), device="cuda")
+        torch.cuda.synchronize()
+        return q, k, v, out
+
+    def run_decode(self, steps, warmup):
+        """Consecutive decode steps appending to the cache."""
+        torch, ctx = self.torch, self.ctx
+        total = warmup + 2 * steps
+        self.alloc(total + 1)
+        q, k, v, out = self.rows(min(total, 64))
+        nt = [1] * self.B
+        n = q.shape[0]
+
+        def step(i):
+            ctx.forward(self.cache, q[i % n], k[i % n], v[i % n], nt, out=out)
+
+        for i in range(warmup):
+            step(i)
+        ctx.sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(warmup + i)
+        ctx.sync()
+        wall = time.perf_counter() - t0
+        # second pass with HIP events around the split-K kernel only
+        ctx.profile(True)
+        for i in range(steps):
+            step(warmup + steps + i)
+        k_ms, launches = ctx.profile_read()
+        ctx.profile(False)
+        vis_wall = [[L + warmup + i + 1 for L in self.lens] for i in range(steps)]
+        vis_prof = [[L + warmup + steps + i + 1 for L in self.lens] for i in range(steps)]
+        b_wall = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_wall) / steps
+        b_prof = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_prof) / steps
+        us = wall / steps * 1e6
+        kus = k_ms / max(launches, 1) * 1e3
+        return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "launches": launches,
+                "bytes_per_step": b_wall, "step_gbps": b_wall / us / 1e3, "kernel_gbps": b_prof / kus / 1e3,
+                "kernel_bytes": b_prof}
+
+    def run_prefill(self, steps, warmup):
+        """T new rows on top of S cached ones; the cache is truncated back between steps."""
+        torch, ctx = self.torch, self.ctx
+        self.alloc(self.T + 1)
+        q, k, v, out = self.rows(1)
+        nt = [self.T] * self.B
+
+        def step():
+            for s, L in enumerate(self.lens):
+                self.cache.truncate(s, L)
+            ctx.forward(self.cache, q[0], k[0], v[0], nt, out=out)
+
+        for _ in range(warmup):
+            step()
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        ctx.sync()
+        wall = time.perf_counter() - t0
+        ctx.profile(True)
+        for _ in range(steps):
+            step()
+        k_ms, launches = ctx.profile_read()
+        ctx.profile(False)
+        fl = sum(prefill_flops(self.H, self.hd, L, self.T) for L in self.lens)
+        us = wall / steps * 1e6
+        kus = k_ms / max(launches, 1) * 1e3
+        return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "launches": launches, "flops": fl,
+                "step_tflops": fl / us / 1e6, "kernel_tflops": fl / kus / 1e6}
+
+    def close(self):
+        if self.cache is not None:
+            self.cache.close()
+        self.ctx.close()
+        self.torch.cuda.empty_cache()
+
+
+def cpu_baseline(w, reps):
+    """The oracle (C restatement of the reference's scalar CPU path), one thread, on one
+    decode layer-step of the headline workload: same shapes, same cache contents."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    blocks = []
+    for s in range(w.B):
+        b = orc.Block(w.H * w.hd, w.H, w.KV, w.hd, eps=1e-6, rope_theta=w.theta)
+        if w.qn is not None:
+            b.set_qk_norm(w.qn, w.kn)
+        n = w.cache.len(s)
+        kv = [w.cache.read(s, c, 0, n) for c in range(w.KV)]
+        b.fill_cache(np.stack([x[0] for x in kv]), np.stack([x[1] for x in kv]))
+        blocks.append(b)
+    r = np.random.default_rng(0)
+    times = []
+    for _ in range(reps):
+        rows = [tuple(r.standard_normal((1, n_ * w.hd)).astype(np.float32) for n_ in (w.H, w.KV, w.KV))
+                for _ in blocks]
+        t0 = time.perf_counter()
+        for b, (q, k, v) in zip(blocks, rows):
+            b.attention_cached_qkv(q, k, v, threads=1)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2] * 1e6
+
+
+def load_traffic(kernel, workload):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept as a
+    committed summary; None until measured."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel, {}).get(workload)
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on one GPU only (sequences, kv heads and context "
+              "slices shard without communication inside attention); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import shainet_amd as sa
+
+    if not sa.HIP.fully_available():
+        print("bench.py: no gfx950 device or libshainet_hip_kernels.so missing (no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+
+    K, W = args.steps, args.warmup
+    only = set(filter(None, args.only.split(",")))
+    lens3 = [int(x) for x in np.random.default_rng(2024).integers(2048, 8193, 16)]
+    results = {}
+
+    def want(name):
+        return not only or name in only
+
+    # headline: configs[2]
+    head = Workload(sa, torch, "qwen3_8b_decode_b16_ctx2048-8192", 32, 8, 128, 1e6, True, lens3, 1, 3)
+    results[head.name] = head.run_decode(K, W)
+    cpu = None
+    if not args.no_cpu:
+        cpu_us = cpu_baseline(head, 5)
+        cpu = {"value": cpu_us, "unit": "us/layer-step", "cores": 1, "kind": "port",
+               "sample": "one decode layer-step of the headline workload (16 sequences, same cache), "
+                         "median of 5, C restatement of the reference's single-threaded Crystal path",
+               "host_cores_visible": os.cpu_count()}
+    head.close()
+
+    small = max(10, K // 4)
+    decode_cfgs = [
+        ("llama1b_decode_b1_ctx1024", 32, 8, 64, 5e5, False, [1024], K),
+        ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096], K),
+        ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384], K),
+        ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4, K),
+    ]
+    for name, H, KV, hd, th, norm, lens, k_ in decode_cfgs:
+        if want(name):
+            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, 1, 5)
+            results[name] = w.run_decode(k_, W)
+            w.close()
+    prefill_cfgs = [
+        ("llama1b_prefill_t2048", 32, 8, 64, 5e5, False, [0], 2048, small),
+        ("llama1b_prefill_t8192", 32, 8, 64, 5e5, False, [0], 8192, max(5, K // 20)),
+        ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512, max(5, K // 10)),
+    ]
+    for name, H, KV, hd, th, norm, lens, T, k_ in prefill_cfgs:
+        if want(name):
+            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, T, 7)
+            results[name] = w.run_prefill(k_, max(2, W // 4))
+            w.close()
+
+    h = results[head.name]
+    line = {
+        "metric": "decode attn us/layer-step (achieved HBM GB/s and prefill TFLOP/s alongside)",
+        "value": round(h["us_per_step"], 3),
+        "unit": "us/layer-step",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(h["us_per_step"] / 1e3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": head.name, "num_heads": 32, "num_kv_heads": 8, "head_dim": 128, "qk_norm": True,
+                   "rope_theta": 1e6, "batch": 16, "cached_lengths": lens3, "new_rows_per_sequence": 1},
+        "hbm_gbps": round(h["step_gbps"], 1),
+        "roofline": {"bound": "hbm", "kernel": "decode_splitk_kernel<128>", "achieved": round(h["kernel_gbps"], 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(h["kernel_gbps"] / HBM_PEAK_GBPS, 4),
+                     "kernel_us": round(h["kernel_us"], 2), "bytes_per_launch": int(h["kernel_bytes"]),
+                     "traffic": load_traffic("decode_splitk_kernel<128>", head.name)},
+        "cpu_baseline": cpu,
+        "workloads": {k_: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in r.items()
+                           if kk != "workload"} for k_, r in results.items()},
+    }
+    p = results.get("llama1b_prefill_t2048")
+    if p:
+        line["prefill_tflops"] = round(p["step_tflops"], 2)
+        line["roofline_prefill"] = {"bound": "mfma", "kernel": "prefill_mfma_kernel<64>", "workload": p["workload"],
+                                    "achieved": round(p["kernel_tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
+                                    "unit": "TFLOP/s", "frac": round(p["kernel_tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
+                                    "kernel_us": round(p["kernel_us"], 2), "flops_per_launch": p["flops"],
+                                    "traffic": load_traffic("prefill_mfma_kernel<64>", p["workload"])}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

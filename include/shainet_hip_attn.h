@@ -108,6 +108,10 @@ int shainet_kv_cache_destroy(shainet_kv_cache *cache);
  * clears every sequence. */
 int shainet_kv_cache_clear(shainet_kv_cache *cache, int seq);
 
+/* Drop the rows at positions >= len of one sequence (len <= its current length):
+ * regenerate from an earlier point without refilling.  clear is truncate to 0. */
+int shainet_kv_cache_truncate(shainet_kv_cache *cache, int seq, int len);
+
 /* Number of cached positions of one sequence (@cache_len, llama_block.cr:48), or -1. */
 int shainet_kv_cache_len(const shainet_kv_cache *cache, int seq);
 int shainet_kv_cache_capacity(const shainet_kv_cache *cache);
@@ -151,6 +155,23 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
  * ([sum new_tokens, num_heads*head_dim], host): lets a test check RoPE positions
  * and QK-norm of Q exactly (llama_block.cr:332-344). */
 int shainet_attn_last_q_rot(shainet_attn_ctx *ctx, float *out, int rows);
+
+/* Kernel timing for benchmarks: while enabled, every shainet_attn_forward call
+ * brackets its attention kernel (the split-K decode kernel, the MFMA prefill
+ * kernel or the generic kernel; not the prep or combine kernels) with HIP events
+ * on the context's stream.  shainet_attn_profile_read waits for the stream,
+ * returns the summed kernel time in milliseconds and the number of launches
+ * since the last read, and resets both.  No counterpart in the reference. */
+int shainet_attn_profile(shainet_attn_ctx *ctx, int enable);
+int shainet_attn_profile_read(shainet_attn_ctx *ctx, double *total_ms, int *launches);
+
+/* Plain streaming kernels of known size (device pointers, n floats, n % 4 == 0,
+ * grid-stride over `workgroups` workgroups of 256 lanes, on `stream`): a copy
+ * and a read that writes one float per workgroup into sink[workgroups].  They
+ * calibrate the HBM byte counters and the reachable stream bandwidth that the
+ * attention kernels are compared with.  No counterpart in the reference. */
+int shainet_hip_stream_copy_f32(const float *src, float *dst, long long n, int workgroups, void *stream);
+int shainet_hip_stream_read_f32(const float *src, float *sink, long long n, int workgroups, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,15 +1,9 @@
 // Causal grouped-query attention over the device KV cache for gfx950 (CDNA4).
 //
-// Three kernels replace attention_heads_cpu (llama_block.cr:302-401) and the
-// reference's attention_kv_kernel (cuda_kernels.cu:734-806):
+// Together with decode_kernel.hip (one new row per sequence) these kernels replace
+// attention_heads_cpu (llama_block.cr:302-401) and the reference's
+// attention_kv_kernel (cuda_kernels.cu:734-806):
 //
-//   decode_splitk_kernel  one new row per sequence.  Split-K over the cached
-//       positions: every wavefront streams 16-key tiles of K and V straight from
-//       HBM into MFMA operands (v_mfma_f32_16x16x4_f32, the g query heads of a
-//       GQA group are the tile's columns, so K and V are read once per group),
-//       keeps an online softmax, and the four wavefronts of a workgroup merge
-//       their (max, sum, O) through LDS.  A second small kernel merges the
-//       workgroups of one sequence.
 //   prefill_mfma_kernel   many new rows.  Query rows and the heads of a group
 //       are flattened into "virtual rows"; a wavefront owns 32 of them, a
 //       workgroup 128.  K/V tiles of 32 keys are staged through LDS (double
@@ -17,7 +11,7 @@
 //   generic_attn_kernel   any head_dim; one wavefront per (row, head).  Used for
 //       head dims other than 64 and 128.
 //
-// All three compute S^T = K Q^T so that the probabilities come out of the MFMA
+// The MFMA kernels compute S^T = K Q^T so that the probabilities come out of the MFMA
 // accumulator already laid out as the B operand of O^T = V^T P^T: no transpose,
 // no LDS round trip for P.  The contraction index of an MFMA may be visited in
 // any order as long as A and B agree, which lets every lane fetch 16-byte
@@ -39,177 +33,6 @@ __device__ __forceinline__ int find_seq(const SeqTable &st, int item, const int 
   int s = 0;
   while (s + 1 < st.n_seqs && item >= off[s + 1]) ++s;
   return s;
-}
-
-// ---------------------------------------------------------------------------
-// Decode: split-K, one new row per sequence.
-//
-// MFMA 16x16x4 operand layout (lane l): A[m = l%16][k = l/16], B[k = l/16][n = l%16],
-// D[m = 4*(l/16) + r][n = l%16] for accumulator register r = 0..3.
-//   scores:  D = S^T, m = key within the tile, n = query head within the group.
-//            K-step s of lane group j = l/16 covers d = 16*(s/4) + 4*j + s%4, so
-//            a lane fetches K as float4 at offsets 16*i + 4*j of its key row.
-//   output:  D = O^T tile t, m = d index, n = head; the contraction runs over the
-//            tile's keys, k-step r of lane group j is key 4*j + r, which is exactly
-//            where accumulator register r of S^T lives.  Row m of tile t is
-//            d = NT*m + t, so a lane fetches NT consecutive floats of a V row.
-template <int HD>
-__global__ __launch_bounds__(256) void decode_splitk_kernel(const float *__restrict__ q_rot,
-                                                            const float *__restrict__ kc,
-                                                            const float *__restrict__ vc,
-                                                            float *__restrict__ out,
-                                                            float *__restrict__ part_o,
-                                                            float *__restrict__ part_ml, SeqTable st,
-                                                            Shape sh, int chunk, float c) {
-  constexpr int NT = HD / 16;  // float4 loads per lane per K tile; d tiles of the output
-  extern __shared__ float smem[];
-  const int item = blockIdx.x, kvh = blockIdx.y;
-  const int s = find_seq(st, item, st.work_off);
-  const int ci = item - st.work_off[s];
-  const int n_chunks = st.work_off[s + 1] - st.work_off[s];
-  const int L = st.start_pos[s] + 1;  // visible keys of the one new row
-  const int k_begin = ci * chunk;
-  const int k_end = min(L, k_begin + chunk);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col = lane & 15, j = lane >> 4;
-  const int g = sh.g;
-  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
-  const float *kbase = kc + head_base;
-  const float *vbase = vc + head_base;
-  const int token = st.tok_off[s];
-
-  float qr[HD / 4];
-  {
-    const float *qp = q_rot + ((long long)token * sh.H + kvh * g + (col < g ? col : 0)) * HD + 4 * j;
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-      f32x4 t = *(const f32x4 *)(qp + 16 * i);
-      if (col >= g) t = f32x4{0.f, 0.f, 0.f, 0.f};
-      qr[4 * i + 0] = t.x;
-      qr[4 * i + 1] = t.y;
-      qr[4 * i + 2] = t.z;
-      qr[4 * i + 3] = t.w;
-    }
-  }
-
-  float m = -INFINITY, l = 0.f;
-  f32x4 o[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  for (int kb = k_begin + wave * 16; kb < k_end; kb += 64) {
-    // rows past the end are clamped to the last valid row: finite data, weight 0
-    const float *kp = kbase + (long long)min(kb + col, L - 1) * HD + 4 * j;
-    f32x4 kr[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) kr[i] = *(const f32x4 *)(kp + 16 * i);
-    float vr[4][NT];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float *vp = vbase + (long long)min(kb + 4 * j + r, L - 1) * HD + NT * col;
-#pragma unroll
-      for (int i = 0; i < NT / 4; ++i) {
-        f32x4 t = *(const f32x4 *)(vp + 4 * i);
-        vr[r][4 * i + 0] = t.x;
-        vr[r][4 * i + 1] = t.y;
-        vr[r][4 * i + 2] = t.z;
-        vr[r][4 * i + 3] = t.w;
-      }
-    }
-
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-      s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].x, qr[4 * i + 0], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].y, qr[4 * i + 1], s1, 0, 0, 0);
-      s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].z, qr[4 * i + 2], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[i].w, qr[4 * i + 3], s1, 0, 0, 0);
-    }
-    float sv[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) sv[r] = (kb + 4 * j + r < k_end) ? s0[r] + s1[r] : -INFINITY;
-    float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mnew = fmaxf(m, mx);  // finite: key kb is valid
-    const float alpha = fast_exp2((m - mnew) * c);
-    float p[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) p[r] = fast_exp2((sv[r] - mnew) * c);
-    l = l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
-    m = mnew;
-#pragma unroll
-    for (int t = 0; t < NT; ++t) o[t] *= alpha;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) o[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[r][t], p[r], o[t], 0, 0, 0);
-  }
-
-  // merge the four wavefronts through LDS: sm_o[wave][col][d], sm_m/sm_l[wave][col]
-  l += __shfl_xor(l, 16);
-  l += __shfl_xor(l, 32);
-  float *sm_o = smem;
-  float *sm_m = smem + 4 * g * HD;
-  float *sm_l = sm_m + 4 * g;
-  if (col < g) {
-    float *dst = sm_o + (wave * g + col) * HD;
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) dst[NT * (4 * j + r) + t] = o[t][r];
-    if (j == 0) {
-      sm_m[wave * g + col] = m;
-      sm_l[wave * g + col] = l;
-    }
-  }
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < g * HD; idx += 256) {
-    const int cc = idx / HD, d = idx - cc * HD;
-    float mm = sm_m[cc];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w * g + cc]);
-    float acc = 0.f, ls = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float f = fast_exp2((sm_m[w * g + cc] - mm) * c);  // 0 for a wavefront that saw no key
-      acc += f * sm_o[(w * g + cc) * HD + d];
-      ls += f * sm_l[w * g + cc];
-    }
-    const int h = kvh * g + cc;
-    if (n_chunks == 1) {
-      out[((long long)token * sh.H + h) * HD + d] = acc / ls;
-    } else {
-      const long long pi = ((long long)item * sh.KV + kvh) * g + cc;
-      part_o[pi * HD + d] = acc;
-      if (d == 0) {
-        part_ml[2 * pi] = mm;
-        part_ml[2 * pi + 1] = ls;
-      }
-    }
-  }
-}
-
-// Merge the split-K partials of one (sequence, head): online-softmax combine.
-__global__ void decode_combine_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
-                                      float *__restrict__ out, SeqTable st, Shape sh, float c) {
-  const int s = blockIdx.x, h = blockIdx.y;
-  const int first = st.work_off[s], n = st.work_off[s + 1] - first;
-  if (n <= 1) return;  // written by the split kernel itself
-  const int kvh = h / sh.g, cc = h - kvh * sh.g;
-  const int hd = sh.hd;
-  float mm = -INFINITY;
-  for (int i = 0; i < n; ++i) mm = fmaxf(mm, part_ml[2 * ((((long long)(first + i)) * sh.KV + kvh) * sh.g + cc)]);
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float acc = 0.f, ls = 0.f;
-    for (int i = 0; i < n; ++i) {
-      const long long pi = (((long long)(first + i)) * sh.KV + kvh) * sh.g + cc;
-      const float f = fast_exp2((part_ml[2 * pi] - mm) * c);
-      acc += f * part_o[pi * hd + d];
-      ls += f * part_ml[2 * pi + 1];
-    }
-    out[((long long)st.tok_off[s] * sh.H + h) * hd + d] = acc / ls;
-  }
 }
 
 // ---------------------------------------------------------------------------
@@ -459,24 +282,11 @@ Path choose_path(const SeqTable &st, const Shape &sh) {
   return Path::kPrefillMfma;
 }
 
-int choose_decode_chunk(const SeqTable &st, const Shape &sh) {
-  long long keys = 0;
-  for (int s = 0; s < st.n_seqs; ++s) keys += st.start_pos[s] + 1;
-  // aim for about eight workgroups per compute unit over the whole launch
-  long long chunk = (keys * sh.KV + 2047) / 2048;
-  chunk = (chunk + 63) / 64 * 64;
-  if (chunk < 64) chunk = 64;
-  if (chunk > 1024) chunk = 1024;
-  return (int)chunk;
-}
-
-int plan_work(SeqTable &st, const Shape &sh, Path path, int decode_chunk) {
+int plan_work(SeqTable &st, const Shape &sh, Path path) {
   st.work_off[0] = 0;
   for (int s = 0; s < st.n_seqs; ++s) {
     int items;
-    if (path == Path::kDecodeSplitK)
-      items = (st.start_pos[s] + 1 + decode_chunk - 1) / decode_chunk;
-    else if (path == Path::kPrefillMfma)
+    if (path == Path::kPrefillMfma)
       items = (st.n_new[s] * sh.g + 127) / 128;
     else
       items = st.n_new[s];
@@ -485,44 +295,12 @@ int plan_work(SeqTable &st, const Shape &sh, Path path, int decode_chunk) {
   return st.work_off[st.n_seqs];
 }
 
-size_t decode_partial_floats(const Shape &sh, int items) {
-  return (size_t)items * sh.KV * sh.g * (sh.hd + 2);
-}
-
 static bool table_ok(const SeqTable &st, const Shape &sh) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.H != sh.KV * sh.g) return false;
   for (int s = 0; s < st.n_seqs; ++s)
     if (st.n_new[s] < 1 || st.start_pos[s] < 0 || st.start_pos[s] + st.n_new[s] > sh.cap || st.slot[s] < 0)
       return false;
   return true;
-}
-
-hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
-                         const SeqTable &st, const Shape &sh, int items, int decode_chunk, float scale,
-                         hipStream_t stream) {
-  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || sh.g > 16 || decode_chunk % 64 || items < 1)
-    return hipErrorInvalidValue;
-  for (int s = 0; s < st.n_seqs; ++s)
-    if (st.n_new[s] != 1) return hipErrorInvalidValue;
-  float *part_o = partials;
-  float *part_ml = partials + (size_t)items * sh.KV * sh.g * sh.hd;
-  const float c = scale * kLog2e;
-  const size_t smem = (size_t)(4 * sh.g * sh.hd + 8 * sh.g) * sizeof(float);
-  dim3 grid((unsigned)items, (unsigned)sh.KV);
-  if (sh.hd == 64)
-    hipLaunchKernelGGL(decode_splitk_kernel<64>, grid, dim3(256), smem, stream, q_rot, kc, vc, out, part_o, part_ml,
-                       st, sh, decode_chunk, c);
-  else
-    hipLaunchKernelGGL(decode_splitk_kernel<128>, grid, dim3(256), smem, stream, q_rot, kc, vc, out, part_o,
-                       part_ml, st, sh, decode_chunk, c);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  if (items > st.n_seqs) {  // some sequence was split
-    hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)st.n_seqs, (unsigned)sh.H), dim3(sh.hd), 0, stream,
-                       part_o, part_ml, out, st, sh, c);
-    e = hipGetLastError();
-  }
-  return e;
 }
 
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,

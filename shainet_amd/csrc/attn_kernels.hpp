@@ -42,17 +42,23 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
 enum class Path { kDecodeSplitK, kPrefillMfma, kGeneric };
 Path choose_path(const SeqTable &st, const Shape &sh);
 
-// Fills st.work_off for the chosen path and returns the number of work items.
-// decode_chunk is the number of keys one decode workgroup covers (multiple of 64).
-int plan_work(SeqTable &st, const Shape &sh, Path path, int decode_chunk);
-int choose_decode_chunk(const SeqTable &st, const Shape &sh);
+// Fills st.work_off for the prefill or generic path and returns the number of work items.
+int plan_work(SeqTable &st, const Shape &sh, Path path);
 
-// Floats needed for split-K partials of a decode call with `items` work items.
-size_t decode_partial_floats(const Shape &sh, int items);
+// Decode work split: the 16-key tiles of all (sequence, kv head) pairs laid end to
+// end (st.work_off = per-sequence prefix sums) and cut into equal spans.
+struct DecodePlan {
+  int total_tiles;
+  int tiles_per_wg;
+  int n_wgs;
+  int n_slots;  // partial slots: workgroup index + pair index is unique per segment
+};
+DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
+size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 
 hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
-                         const SeqTable &st, const Shape &sh, int items, int decode_chunk, float scale,
-                         hipStream_t stream);
+                         const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
+                         hipStream_t stream, hipEvent_t before_split = nullptr, hipEvent_t after_split = nullptr);
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
                           const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream);
 hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,

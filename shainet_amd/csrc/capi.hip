@@ -79,7 +79,9 @@ struct shainet_attn_ctx {
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
   int last_rows = 0;
-  int decode_chunk_override = 0;
+  int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
+  bool profiling = false;
+  std::vector<hipEvent_t> prof_events;  // start, stop, start, stop, ...
 };
 
 struct shainet_kv_cache {
@@ -151,18 +153,28 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, const float *kc, cons
                   SeqTable &st, const Shape &sh, int total_tokens, float scale, hipStream_t stream) {
   const Path path = choose_path(st, sh);
   hipError_t e;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  if (c->profiling) {
+    if (hipEventCreate(&ev0) != hipSuccess || hipEventCreate(&ev1) != hipSuccess)
+      return fail(SHAINET_HIP_ERR_RUNTIME, "hipEventCreate failed");
+    c->prof_events.push_back(ev0);
+    c->prof_events.push_back(ev1);
+  }
   if (path == Path::kDecodeSplitK) {
-    const int chunk = c->decode_chunk_override ? c->decode_chunk_override : choose_decode_chunk(st, sh);
-    const int items = plan_work(st, sh, path, chunk);
-    int rc = c->partials.reserve(decode_partial_floats(sh, items));
+    const DecodePlan plan = plan_decode(st, sh, c->decode_wgs_override);
+    int rc = c->partials.reserve(decode_partial_floats(sh, plan));
     if (rc) return rc;
-    e = launch_decode(q_rot, kc, vc, out, c->partials.p, st, sh, items, chunk, scale, stream);
+    e = launch_decode(q_rot, kc, vc, out, c->partials.p, st, sh, plan, scale, stream, ev0, ev1);
   } else if (path == Path::kPrefillMfma) {
-    const int items = plan_work(st, sh, path, 0);
+    const int items = plan_work(st, sh, path);
+    if (ev0) (void)hipEventRecord(ev0, stream);
     e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream);
+    if (ev1) (void)hipEventRecord(ev1, stream);
   } else {
-    plan_work(st, sh, path, 0);
+    plan_work(st, sh, path);
+    if (ev0) (void)hipEventRecord(ev0, stream);
     e = launch_generic(q_rot, kc, vc, out, st, sh, total_tokens, scale, stream);
+    if (ev1) (void)hipEventRecord(ev1, stream);
   }
   if (e != hipSuccess) return hip_fail(e, "attention launch");
   return SHAINET_HIP_OK;
@@ -253,9 +265,9 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
   c->inv_freq.resize(head_dim / 2);
   for (int i = 0; i < head_dim / 2; ++i)  // llama_block.cr:669-675
     c->inv_freq[i] = rope_freqs ? rope_freqs[i] : (float)(1.0 / pow(rope_theta, 2.0 * i / head_dim));
-  if (const char *env = getenv("SHAINET_HIP_DECODE_CHUNK")) {
+  if (const char *env = getenv("SHAINET_HIP_DECODE_WGS")) {  // tuning knob: workgroups of the decode split
     int v = atoi(env);
-    if (v >= 64 && v % 64 == 0) c->decode_chunk_override = v;
+    if (v >= 1 && v <= 65536) c->decode_wgs_override = v;
   }
   int rc = SHAINET_HIP_OK;
   hipError_t e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
@@ -299,6 +311,7 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
   for (float *p : {c->d_q_norm, c->d_k_norm, c->d_bq, c->d_bk, c->d_bv})
     if (p) (void)hipFree(p);
   if (c->d_rope) (void)hipFree(c->d_rope);
+  for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
   delete c;
   return SHAINET_HIP_OK;
@@ -365,6 +378,14 @@ int shainet_kv_cache_clear(shainet_kv_cache *kc, int seq) {
     kc->len.assign(kc->batch, 0);
   else
     kc->len[seq] = 0;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_kv_cache_truncate(shainet_kv_cache *kc, int seq, int len) {
+  if (!kc || seq < 0 || seq >= kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid sequence");
+  if (len < 0 || len > kc->len[seq])
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "truncate to %d outside 0..%d", len, kc->len[seq]);
+  kc->len[seq] = len;
   return SHAINET_HIP_OK;
 }
 
@@ -520,6 +541,33 @@ int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *s
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
   }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_profile(shainet_attn_ctx *c, int enable) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
+  c->profiling = enable != 0;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_profile_read(shainet_attn_ctx *c, double *total_ms, int *launches) {
+  if (!c || !total_ms || !launches) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  double sum = 0.0;
+  int n = 0;
+  for (size_t i = 0; i + 1 < c->prof_events.size(); i += 2) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, c->prof_events[i], c->prof_events[i + 1]) == hipSuccess) {
+      sum += ms;
+      ++n;
+    }
+    (void)hipEventDestroy(c->prof_events[i]);
+    (void)hipEventDestroy(c->prof_events[i + 1]);
+  }
+  (void)hipGetLastError();
+  c->prof_events.clear();
+  *total_ms = sum;
+  *launches = n;
   return SHAINET_HIP_OK;
 }
 

@@ -1,0 +1,354 @@
+// Split-K (flash-decoding) attention of one new row per sequence over the device
+// KV cache, for gfx950.  Replaces the T = 1 case of attention_heads_cpu
+// (llama_block.cr:302-401) and of the reference's attention_kv_kernel
+// (cuda_kernels.cu:734-806), which launches one block per query head and walks
+// the keys serially.
+//
+// Work split.  The key ranges of all (sequence, kv head) pairs are laid end to
+// end in units of 16-key tiles and cut into equal contiguous spans, one per
+// workgroup, so every workgroup streams the same number of bytes whatever the
+// sequence lengths are.  A span that crosses a pair boundary is processed as two
+// segments.  The four wavefronts of a workgroup take the tiles of a segment
+// round-robin, each keeping its own online softmax, and merge through LDS into
+// one partial (max, sum, O) per segment; a second kernel merges the partials of
+// each pair.
+//
+// Per 16-key tile a wavefront
+//   * copies the K tile (16 contiguous rows) from HBM straight into LDS with
+//     global_load_lds_dwordx4, 1 KiB per instruction, fully coalesced, with the
+//     16-byte pieces of each row XOR-swizzled so that the later ds_read_b128 of
+//     MFMA operands is bank-conflict free;
+//   * loads the V tile into registers (256 contiguous bytes per 16 lanes);
+//   * computes S^T = K Q^T with v_mfma_f32_16x16x4_f32: rows = keys, columns =
+//     the g query heads of the GQA group, so K and V are read once per group;
+//   * updates the online softmax with wavefront shuffles, and accumulates
+//     O^T += V^T P^T with the probabilities taken directly from the S^T
+//     accumulator registers (they already have the B-operand layout).
+// The loads of tile t+1 are issued before the arithmetic of tile t.
+//
+// MFMA 16x16x4 operand layout (lane l): A[m = l%16][k = l/16], B[k = l/16][n = l%16],
+// D[m = 4*(l/16) + r][n = l%16] for accumulator register r = 0..3.  The
+// contraction index may be visited in any order as long as A and B agree:
+//   scores: k-step s of lane group j = l/16 covers d = 16*(s/4) + 4*j + s%4;
+//   output: tile t, row m is d = 64*(t/4) + 4*m + t%4; k-step r of lane group j is
+//           key 4*j + r of the tile, where accumulator register r of S^T lives.
+#include "attn_kernels.hpp"
+
+#include <math.h>
+#include <stdint.h>
+
+namespace shainet {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(uintptr_t)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+
+template <int HD>
+struct DecodeCfg {
+  static constexpr int NT = HD / 16;         // float4 of K per lane per tile; d tiles of the output
+  static constexpr int PPR = HD / 4;         // 16-byte pieces per row
+  static constexpr int ROW_BYTES = HD * 4;
+  static constexpr int TILE_BYTES = 16 * ROW_BYTES;
+  static constexpr int NKI = TILE_BYTES / 1024;  // global_load_lds instructions per K tile
+  static constexpr int NVU = HD / 64;            // float4 of a V row per lane
+};
+
+// Issue the asynchronous copy of the K tile starting at row `kb` into `lds`.
+template <int HD>
+__device__ __forceinline__ void issue_k_tile(const float *kbase, int kb, int last_row, char *lds, int lane) {
+  using C = DecodeCfg<HD>;
+#pragma unroll
+  for (int u = 0; u < C::NKI; ++u) {
+    const int slot = u * 64 + lane;
+    const int row = slot / C::PPR, q = slot % C::PPR;
+    const int piece = q ^ row;  // row < 16 only touches the low four bits
+    const float *src = kbase + (long long)min(kb + row, last_row) * HD + 4 * piece;
+    __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src), LDS_PTR(lds + u * 1024), 16, 0, 0);
+  }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last_row, int col, int j,
+                                            f32x4 (&v)[4][DecodeCfg<HD>::NVU]) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float *vp = vbase + (long long)min(kb + 4 * j + r, last_row) * HD + 4 * col;
+#pragma unroll
+    for (int u = 0; u < DecodeCfg<HD>::NVU; ++u) v[r][u] = *(const f32x4 *)(vp + 64 * u);
+  }
+}
+
+template <int HD>
+__global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__restrict__ q_rot,
+                                                               const float *__restrict__ kc,
+                                                               const float *__restrict__ vc,
+                                                               float *__restrict__ out,
+                                                               float *__restrict__ part_o,
+                                                               float *__restrict__ part_ml, SeqTable st,
+                                                               Shape sh, int tiles_per_wg, int total_tiles,
+                                                               int n_slots, float c) {
+  using C = DecodeCfg<HD>;
+  constexpr int NT = C::NT;
+  __shared__ __attribute__((aligned(1024))) char k_lds[4][2][C::TILE_BYTES];
+  extern __shared__ float merge_lds[];  // [4][g][HD] O, [4][g] max, [4][g] sum
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, j = lane >> 4;
+  const int g = sh.g;
+  const int t_begin = blockIdx.x * tiles_per_wg;
+  const int t_end = min(total_tiles, t_begin + tiles_per_wg);
+  char *my_lds = &k_lds[wave][0][0];
+
+  int t = t_begin;
+  int s = 0;
+  while (t < t_end) {
+    while (s + 1 < st.n_seqs && t >= st.work_off[s + 1]) ++s;
+    const int L = st.start_pos[s] + 1;  // visible keys of the one new row
+    const int n_s = (L + 15) >> 4;      // tiles per kv head of this sequence
+    const int rel = t - st.work_off[s];
+    const int kvh = rel / n_s, tile0 = rel - kvh * n_s;
+    const int seg_tiles = min(n_s - tile0, t_end - t);
+    const int tile1 = tile0 + seg_tiles;
+    const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
+    const float *kbase = kc + head_base;
+    const float *vbase = vc + head_base;
+    const int token = st.tok_off[s];
+
+    float qr[HD / 4];
+    {
+      const float *qp = q_rot + ((long long)token * sh.H + kvh * g + (col < g ? col : 0)) * HD + 4 * j;
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        f32x4 x = *(const f32x4 *)(qp + 16 * i);
+        if (col >= g) x = f32x4{0.f, 0.f, 0.f, 0.f};
+        qr[4 * i + 0] = x.x;
+        qr[4 * i + 1] = x.y;
+        qr[4 * i + 2] = x.z;
+        qr[4 * i + 3] = x.w;
+      }
+    }
+
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    f32x4 v_next[4][C::NVU];
+    int tile = tile0 + wave;
+    if (tile < tile1) {
+      issue_k_tile<HD>(kbase, tile * 16, L - 1, my_lds, lane);
+      load_v_tile<HD>(vbase, tile * 16, L - 1, col, j, v_next);
+    }
+    for (int it = 0; tile < tile1; tile += 4, ++it) {
+      const int kb = tile * 16;
+      char *buf = my_lds + (it & 1) * C::TILE_BYTES;
+      // everything issued so far (this tile's K copy and V loads) has landed:
+      // s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima), then a
+      // compiler barrier so that no LDS read of the tile is scheduled above it
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      asm volatile("" ::: "memory");
+      f32x4 v_cur[4][C::NVU];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int u = 0; u < C::NVU; ++u) v_cur[r][u] = v_next[r][u];
+      if (tile + 4 < tile1) {
+        issue_k_tile<HD>(kbase, kb + 64, L - 1, my_lds + ((it + 1) & 1) * C::TILE_BYTES, lane);
+        load_v_tile<HD>(vbase, kb + 64, L - 1, col, j, v_next);
+      }
+
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+      const char *krow = buf + col * C::ROW_BYTES;
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const f32x4 kk = *(const f32x4 *)(krow + (((4 * i + j) ^ col) << 4));
+        s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kk.x, qr[4 * i + 0], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kk.y, qr[4 * i + 1], s1, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kk.z, qr[4 * i + 2], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kk.w, qr[4 * i + 3], s1, 0, 0, 0);
+      }
+      float sv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sv[r] = (kb + 4 * j + r < L) ? s0[r] + s1[r] : -INFINITY;
+      float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mnew = fmaxf(m, mx);  // finite: key kb is valid
+      const float alpha = fast_exp2((m - mnew) * c);
+      float p[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p[r] = fast_exp2((sv[r] - mnew) * c);
+      l = l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
+      m = mnew;
+#pragma unroll
+      for (int i = 0; i < NT; ++i) o[i] *= alpha;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int u = 0; u < C::NVU; ++u) {
+          o[4 * u + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(v_cur[r][u].x, p[r], o[4 * u + 0], 0, 0, 0);
+          o[4 * u + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(v_cur[r][u].y, p[r], o[4 * u + 1], 0, 0, 0);
+          o[4 * u + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(v_cur[r][u].z, p[r], o[4 * u + 2], 0, 0, 0);
+          o[4 * u + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(v_cur[r][u].w, p[r], o[4 * u + 3], 0, 0, 0);
+        }
+    }
+
+    // merge the four wavefronts through LDS
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    float *sm_o = merge_lds;
+    float *sm_m = merge_lds + 4 * g * HD;
+    float *sm_l = sm_m + 4 * g;
+    __syncthreads();  // the previous segment's readers are done with merge_lds
+    if (col < g) {
+      float *dst = sm_o + (wave * g + col) * HD;
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[64 * (i >> 2) + 4 * (4 * j + r) + (i & 3)] = o[i][r];
+      if (j == 0) {
+        sm_m[wave * g + col] = m;
+        sm_l[wave * g + col] = l;
+      }
+    }
+    __syncthreads();
+    const bool whole_pair = tile0 == 0 && tile1 == n_s;
+    const int pair = s * sh.KV + kvh;
+    const int slot = blockIdx.x + pair;  // unique: both terms only grow along the tile stream
+    for (int idx = threadIdx.x; idx < g * HD; idx += 256) {
+      const int cc = idx / HD, d = idx - cc * HD;
+      float mm = sm_m[cc];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w * g + cc]);
+      float acc = 0.f, ls = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float f = fast_exp2((sm_m[w * g + cc] - mm) * c);  // 0 for a wavefront that saw no tile
+        acc += f * sm_o[(w * g + cc) * HD + d];
+        ls += f * sm_l[w * g + cc];
+      }
+      if (whole_pair) {
+        out[((long long)token * sh.H + kvh * g + cc) * HD + d] = acc / ls;
+      } else if (slot < n_slots) {
+        const long long pi = (long long)slot * g + cc;
+        part_o[pi * HD + d] = acc;
+        if (d == 0) {
+          part_ml[2 * pi] = mm;
+          part_ml[2 * pi + 1] = ls;
+        }
+      }
+    }
+    t += seg_tiles;
+  }
+}
+
+// Merge the partials of one (sequence, head): one wavefront each.
+__global__ __launch_bounds__(256) void decode_combine_kernel(const float *__restrict__ part_o,
+                                                             const float *__restrict__ part_ml,
+                                                             float *__restrict__ out, SeqTable st, Shape sh,
+                                                             int tiles_per_wg, float c) {
+  const int lane = threadIdx.x & 63;
+  const int id = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (id >= st.n_seqs * sh.H) return;
+  const int s = id / sh.H, h = id - s * sh.H;
+  const int kvh = h / sh.g, cc = h - kvh * sh.g;
+  const int n_s = (st.start_pos[s] + 1 + 15) >> 4;
+  const int a = st.work_off[s] + kvh * n_s;  // the pair's tiles are [a, a + n_s)
+  const int w_lo = a / tiles_per_wg, w_hi = (a + n_s - 1) / tiles_per_wg;
+  if (w_lo == w_hi) return;  // one workgroup held the whole pair and wrote the output itself
+  const int pair = s * sh.KV + kvh;
+  const int n = w_hi - w_lo + 1;
+  const int hd = sh.hd;
+  const long long first = (long long)(w_lo + pair) * sh.g + cc;  // partial of workgroup w is first + (w - w_lo)*g
+
+  float mm = -INFINITY;
+  for (int i = lane; i < n; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * sh.g)]);
+  for (int o = 32; o > 0; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
+  float ls = 0.f;
+  for (int i = lane; i < n; i += 64) {
+    const long long pi = first + (long long)i * sh.g;
+    ls += fast_exp2((part_ml[2 * pi] - mm) * c) * part_ml[2 * pi + 1];
+  }
+  for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
+  const float inv = 1.0f / ls;
+  for (int d = lane; d < hd; d += 64) {
+    float acc = 0.f;
+    int i = 0;
+    for (; i + 4 <= n; i += 4) {  // four independent loads in flight
+      float f[4], x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const long long pi = first + (long long)(i + u) * sh.g;
+        f[u] = part_ml[2 * pi];
+        x[u] = part_o[pi * hd + d];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc += fast_exp2((f[u] - mm) * c) * x[u];
+    }
+    for (; i < n; ++i) {
+      const long long pi = first + (long long)i * sh.g;
+      acc += fast_exp2((part_ml[2 * pi] - mm) * c) * part_o[pi * hd + d];
+    }
+    out[((long long)st.tok_off[s] * sh.H + h) * hd + d] = acc * inv;
+  }
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+}  // namespace
+
+DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
+  DecodePlan p;
+  st.work_off[0] = 0;
+  for (int s = 0; s < st.n_seqs; ++s)
+    st.work_off[s + 1] = st.work_off[s] + sh.KV * ((st.start_pos[s] + 1 + 15) / 16);
+  p.total_tiles = st.work_off[st.n_seqs];
+  if (wg_target < 1) wg_target = 512;  // two workgroups on each of the 256 compute units
+  // at least four tiles (one per wavefront) per workgroup
+  int q = (p.total_tiles + wg_target - 1) / wg_target;
+  if (q < 4) q = 4;
+  p.tiles_per_wg = q;
+  p.n_wgs = (p.total_tiles + q - 1) / q;
+  p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
+  return p;
+}
+
+size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
+  return (size_t)p.n_slots * sh.g * (sh.hd + 2);
+}
+
+hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
+                         const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
+                         hipStream_t stream, hipEvent_t before_split, hipEvent_t after_split) {
+  if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
+      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1)
+    return hipErrorInvalidValue;
+  for (int s = 0; s < st.n_seqs; ++s)
+    if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
+      return hipErrorInvalidValue;
+  float *part_o = partials;
+  float *part_ml = partials + (size_t)p.n_slots * sh.g * sh.hd;
+  const float c = scale * kLog2e;
+  const size_t smem = (size_t)(4 * sh.g * sh.hd + 8 * sh.g) * sizeof(float);
+  if (before_split) (void)hipEventRecord(before_split, stream);
+  if (sh.hd == 64)
+    hipLaunchKernelGGL(decode_splitk_kernel<64>, dim3((unsigned)p.n_wgs), dim3(256), smem, stream, q_rot, kc, vc,
+                       out, part_o, part_ml, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+  else
+    hipLaunchKernelGGL(decode_splitk_kernel<128>, dim3((unsigned)p.n_wgs), dim3(256), smem, stream, q_rot, kc, vc,
+                       out, part_o, part_ml, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+  hipError_t e = hipGetLastError();
+  if (after_split) (void)hipEventRecord(after_split, stream);
+  if (e != hipSuccess) return e;
+  const int waves = st.n_seqs * sh.H;
+  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, part_o,
+                     part_ml, out, st, sh, p.tiles_per_wg, c);
+  return hipGetLastError();
+}
+
+}  // namespace shainet

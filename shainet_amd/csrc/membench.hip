@@ -1,0 +1,53 @@
+// Plain streaming kernels of known size.  They calibrate what the HBM counters of
+// rocprofv3 (FETCH_SIZE, WRITE_SIZE) read per byte moved and what bandwidth a
+// perfectly coalesced stream reaches on the device, the yardsticks the attention
+// kernels' traffic and bandwidth figures are compared with.
+#include <hip/hip_runtime.h>
+
+#include "../../include/shainet_hip_attn.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void copy_f32x4_kernel(const f32x4 *__restrict__ src, f32x4 *__restrict__ dst,
+                                                         long long n4) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
+// Reads everything, writes one float per workgroup.
+__global__ __launch_bounds__(256) void read_f32x4_kernel(const f32x4 *__restrict__ src, float *__restrict__ sink,
+                                                         long long n4) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    const f32x4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc += (a + b) + (c + d);
+  }
+  for (; i < n4; i += stride) acc += src[i];
+  float s = (acc.x + acc.y) + (acc.z + acc.w);
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if ((threadIdx.x & 63) == 0) atomicAdd(&sink[blockIdx.x], s);
+}
+
+}  // namespace
+
+extern "C" {
+
+int shainet_hip_stream_copy_f32(const float *src, float *dst, long long n, int workgroups, void *stream) {
+  if (!src || !dst || n < 0 || (n & 3) || workgroups < 1) return SHAINET_HIP_ERR_ARGUMENT;
+  hipLaunchKernelGGL(copy_f32x4_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
+                     (const f32x4 *)src, (f32x4 *)dst, n / 4);
+  return hipGetLastError() == hipSuccess ? SHAINET_HIP_OK : SHAINET_HIP_ERR_RUNTIME;
+}
+
+int shainet_hip_stream_read_f32(const float *src, float *sink, long long n, int workgroups, void *stream) {
+  if (!src || !sink || n < 0 || (n & 3) || workgroups < 1) return SHAINET_HIP_ERR_ARGUMENT;
+  hipLaunchKernelGGL(read_f32x4_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
+                     (const f32x4 *)src, sink, n / 4);
+  return hipGetLastError() == hipSuccess ? SHAINET_HIP_OK : SHAINET_HIP_ERR_RUNTIME;
+}
+
+}  // extern "C"

@@ -65,12 +65,20 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st,
 
   float inv = 1.0f;
   if (w) {
-    // every lane walks the row in the reference's order; the loads are uniform
+    // The sum of squares must run in the reference's order (d ascending, one fp32
+    // add per element).  The row is fetched once, 64 elements per load, and every
+    // lane then walks it through lane broadcasts, so all lanes hold the same sum.
     float ss = 0.0f;
-    for (int d = 0; d < hd; ++d) {
-      float v = bias ? src[d] + bias[d] : src[d];
-      float sq = v * v;
-      ss = ss + sq;
+    for (int d0 = 0; d0 < hd; d0 += 64) {
+      const int d = d0 + lane;
+      float x = 0.0f;
+      if (d < hd) x = bias ? src[d] + bias[d] : src[d];
+      const int n = min(64, hd - d0);
+      for (int t = 0; t < n; ++t) {
+        const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), t));
+        const float sq = v * v;
+        ss = ss + sq;
+      }
     }
     float mean = ss / (float)hd;
     inv = (float)(1.0 / sqrt((double)mean + a.eps));

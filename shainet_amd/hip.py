@@ -61,6 +61,7 @@ _SIGNATURES = {
     "shainet_kv_cache_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_int]),
     "shainet_kv_cache_destroy": (C.c_int, [C.c_void_p]),
     "shainet_kv_cache_clear": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_kv_cache_truncate": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "shainet_kv_cache_len": (C.c_int, [C.c_void_p, C.c_int]),
     "shainet_kv_cache_capacity": (C.c_int, [C.c_void_p]),
     "shainet_kv_cache_reserve": (C.c_int, [C.c_void_p, C.c_int]),
@@ -71,6 +72,10 @@ _SIGNATURES = {
     "shainet_attn_forward": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_int]),
     "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
+    "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
+    "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
+    "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_attn_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), _i32p]),
 }
 
 
@@ -163,6 +168,16 @@ class HIP:
                                heads_per_kv, head_dim, capacity, scale)
 
 
+def stream_copy(src, dst, workgroups=4096, stream=None):
+    """Plain copy kernel over two torch CUDA float tensors of equal size (n % 4 == 0)."""
+    _check(lib().shainet_hip_stream_copy_f32(_ptr(src), _ptr(dst), src.numel(), workgroups, stream))
+
+
+def stream_read(src, sink, workgroups=4096, stream=None):
+    """Plain read kernel; sink is a float tensor of at least `workgroups` elements."""
+    _check(lib().shainet_hip_stream_read_f32(_ptr(src), _ptr(sink), src.numel(), workgroups, stream))
+
+
 class AttnContext:
     """Attention parameters of one LlamaBlock (llama_block.cr:10-28, 73-108)."""
 
@@ -197,6 +212,15 @@ class AttnContext:
 
     def set_stream(self, stream_ptr):
         _check(lib().shainet_attn_set_stream(self._h, stream_ptr))
+
+    def profile(self, enable):
+        _check(lib().shainet_attn_profile(self._h, 1 if enable else 0))
+
+    def profile_read(self):
+        """(summed attention-kernel milliseconds, launches) since the last read."""
+        ms, n = C.c_double(0), C.c_int(0)
+        _check(lib().shainet_attn_profile_read(self._h, C.byref(ms), C.byref(n)))
+        return ms.value, n.value
 
     def inv_freq(self):
         import numpy as np
@@ -257,6 +281,9 @@ class KVCache:
 
     def clear(self, seq=-1):
         _check(lib().shainet_kv_cache_clear(self._h, seq))
+
+    def truncate(self, seq, length):
+        _check(lib().shainet_kv_cache_truncate(self._h, seq, length))
 
     def len(self, seq=0):
         return lib().shainet_kv_cache_len(self._h, seq)
