@@ -58,10 +58,26 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   __shared__ float Ks[2][32 * KSTR];
   __shared__ float Vs[2][32 * HD];
 
-  const int item = blockIdx.x, kvh = blockIdx.y;
-  const int s = find_seq(st, item, st.work_off);
-  const int nblk = st.work_off[s + 1] - st.work_off[s];
-  const int vb = nblk - 1 - (item - st.work_off[s]);  // longest rows first
+  // Workgroups are numbered so that the hardware dispatcher, which hands them out in
+  // index order, starts the row blocks with the longest key ranges first: level 0
+  // is every sequence's last block, level 1 the one before, and so on; the kv head
+  // is the fastest index, so with 8 kv heads each XCD (index % 8) keeps to one head
+  // and its K/V stay in that XCD's L2.  st.work_off[s] = row blocks of sequence s,
+  // st.ord = sequences by descending block count.
+  const int kvh = blockIdx.x % sh.KV;
+  int rank = blockIdx.x / sh.KV;
+  int s = 0, level = 0;
+  for (int b = st.n_seqs - 1; b >= 0; --b) {  // levels [n_{b+1}, n_b) have b+1 active sequences
+    const int lo = b + 1 < st.n_seqs ? st.work_off[st.ord[b + 1]] : 0;
+    const int cnt = (st.work_off[st.ord[b]] - lo) * (b + 1);
+    if (rank < cnt) {
+      level = lo + rank / (b + 1);
+      s = st.ord[rank % (b + 1)];
+      break;
+    }
+    rank -= cnt;
+  }
+  const int vb = st.work_off[s] - 1 - level;
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
   const int L = S + T, VR = T * g;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -292,7 +308,19 @@ int plan_work(SeqTable &st, const Shape &sh, Path path) {
       items = st.n_new[s];
     st.work_off[s + 1] = st.work_off[s] + items;
   }
-  return st.work_off[st.n_seqs];
+  const int total = st.work_off[st.n_seqs];
+  if (path == Path::kPrefillMfma) {
+    // the prefill kernel wants per-sequence block counts and the sequences sorted by them
+    for (int s = 0; s < st.n_seqs; ++s) st.work_off[s] = st.work_off[s + 1] - st.work_off[s];
+    for (int s = 0; s < st.n_seqs; ++s) st.ord[s] = s;
+    for (int a = 1; a < st.n_seqs; ++a)  // insertion sort, descending, stable
+      for (int b = a; b > 0 && st.work_off[st.ord[b]] > st.work_off[st.ord[b - 1]]; --b) {
+        const int t = st.ord[b];
+        st.ord[b] = st.ord[b - 1];
+        st.ord[b - 1] = t;
+      }
+  }
+  return total;
 }
 
 static bool table_ok(const SeqTable &st, const Shape &sh) {
@@ -304,14 +332,28 @@ static bool table_ok(const SeqTable &st, const Shape &sh) {
 }
 
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
-                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream) {
+                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream,
+                          int wgs_per_cu) {
   if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1) return hipErrorInvalidValue;
+  if ((long long)items * sh.KV > 0x7fffffffLL) return hipErrorInvalidValue;
   const float c = scale * kLog2e;
-  dim3 grid((unsigned)items, (unsigned)sh.KV);
+  dim3 grid((unsigned)(items * sh.KV));
+  // static LDS of the kernel: two stages of a padded K tile and a V tile
+  const size_t static_lds = (size_t)2 * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
+  size_t pad = 0;
+  // With fewer workgroups than three per compute unit everything is resident at
+  // once and the dispatcher cannot balance the triangular work: one workgroup per
+  // compute unit lets it hand the short row blocks to whichever unit finishes first.
+  if (wgs_per_cu == 0 && (long long)items * sh.KV <= 768) wgs_per_cu = 1;
+  if (wgs_per_cu >= 1 && wgs_per_cu <= 3) {
+    const size_t want = (size_t)160 * 1024 / wgs_per_cu;  // one more workgroup would not fit
+    const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
+    if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
+  }
   if (sh.hd == 64)
-    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), 0, stream, q_rot, kc, vc, out, st, sh, c);
+    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, st, sh, c);
   else
-    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), 0, stream, q_rot, kc, vc, out, st, sh, c);
+    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, st, sh, c);
   return hipGetLastError();
 }
 

@@ -15,7 +15,8 @@ struct SeqTable {
   int start_pos[kMaxSeqs];     // cached positions before this call
   int n_new[kMaxSeqs];         // rows appended by this call
   int tok_off[kMaxSeqs + 1];   // prefix sums of n_new
-  int work_off[kMaxSeqs + 1];  // prefix sums of per-sequence work items of the attention kernel
+  int work_off[kMaxSeqs + 1];  // per-path work description (see plan_work / plan_decode)
+  int ord[kMaxSeqs];           // prefill: sequences by descending number of row blocks
 };
 
 struct Shape {
@@ -59,8 +60,11 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                          const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before_split = nullptr, hipEvent_t after_split = nullptr);
+// wgs_per_cu: 0 = default; 1..3 pads the kernel's LDS so that at most that many
+// workgroups share a compute unit (a tuning knob).
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
-                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream);
+                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream,
+                          int wgs_per_cu = 0);
 hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);

@@ -80,6 +80,7 @@ struct shainet_attn_ctx {
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
+  int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
   bool profiling = false;
   std::vector<hipEvent_t> prof_events;  // start, stop, start, stop, ...
 };
@@ -168,7 +169,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, const float *kc, cons
   } else if (path == Path::kPrefillMfma) {
     const int items = plan_work(st, sh, path);
     if (ev0) (void)hipEventRecord(ev0, stream);
-    e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream);
+    e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream, c->prefill_wgs_per_cu);
     if (ev1) (void)hipEventRecord(ev1, stream);
   } else {
     plan_work(st, sh, path);
@@ -269,6 +270,7 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
     int v = atoi(env);
     if (v >= 1 && v <= 65536) c->decode_wgs_override = v;
   }
+  if (const char *env = getenv("SHAINET_HIP_PREFILL_WGS_PER_CU")) c->prefill_wgs_per_cu = atoi(env);
   int rc = SHAINET_HIP_OK;
   hipError_t e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
   if (e != hipSuccess) rc = hip_fail(e, "hipStreamCreate");
