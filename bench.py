@@ -189,6 +189,33 @@ def load_traffic(kernel, workload):
         return None
 
 
+def calibrate(torch, sa, reps):
+    """Plain copy and read kernels over 1 GiB: the bandwidth a perfectly coalesced stream
+    reaches here, and (under rocprofv3 --pmc) what FETCH_SIZE / WRITE_SIZE read per byte."""
+    from shainet_amd import hip
+
+    n = 256 * 1024 * 1024
+    a = torch.randn(n, device="cuda")
+    b = torch.empty_like(a)
+    sink = torch.zeros(8192, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {"bytes_per_launch": {"copy_f32x4_kernel": {"read": 4 * n, "write": 4 * n},
+                                "read_f32x4_kernel": {"read": 4 * n, "write": 4 * 768}}}
+    for name, fn, moved in (("copy_f32x4_kernel", lambda: hip.stream_copy(a, b, 4096, stream), 8 * n),
+                            ("read_f32x4_kernel", lambda: hip.stream_read(a, sink, 768, stream), 4 * n)):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        res[name + "_gbps"] = round(moved / (e0.elapsed_time(e1) / reps) / 1e6, 1)
+    print(json.dumps({"calibration": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -196,6 +223,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="run only the plain copy/read kernels of known size (counter and bandwidth yardstick)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on one GPU only (sequences, kv heads and context "
@@ -210,6 +239,10 @@ def main():
     if not sa.HIP.fully_available():
         print("bench.py: no gfx950 device or libshainet_hip_kernels.so missing (no CPU fallback)", file=sys.stderr)
         sys.exit(1)
+
+    if args.calibrate:
+        calibrate(torch, sa, 10)
+        return
 
     K, W = args.steps, args.warmup
     only = set(filter(None, args.only.split(",")))

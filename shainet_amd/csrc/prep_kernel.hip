@@ -18,47 +18,143 @@ namespace shainet {
 
 namespace {
 
-// One wavefront per (token, head row): H query rows, KV key rows, KV value rows.
-__global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
-  const int lane = threadIdx.x & 63;
-  const int rows_per_token = sh.H + 2 * sh.KV;
-  const long long item = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= (long long)total_tokens * rows_per_token) return;
-  const int token = (int)(item / rows_per_token);
-  const int r = (int)(item - (long long)token * rows_per_token);
-  int s = 0;
-  while (s + 1 < st.n_seqs && token >= st.tok_off[s + 1]) ++s;
-  const int pos = st.start_pos[s] + (token - st.tok_off[s]);
-  const int hd = sh.hd, half = hd >> 1;
-  const int q_dim = sh.H * hd, kv_dim = sh.KV * hd;
-
+struct RowRef {
   const float *src, *bias, *w;
   float *dst;
-  bool rotate = true;
+  int pos;
+  bool rotate, valid;
+};
+
+// Row r of a token: the H query heads, then the KV key heads, then the KV value heads.
+__device__ __forceinline__ RowRef locate_row(const PrepArgs &a, const SeqTable &st, const Shape &sh, int token,
+                                             int r, int total_tokens) {
+  RowRef rr;
+  rr.valid = r < sh.H + 2 * sh.KV;
+  if (!rr.valid) r = 0;
+  int s = token;
+  if (total_tokens != st.n_seqs) {  // not one row per sequence: search the prefix sums
+    s = 0;
+    while (s + 1 < st.n_seqs && token >= st.tok_off[s + 1]) ++s;
+  }
+  rr.pos = st.start_pos[s] + (token - st.tok_off[s]);
+  const int hd = sh.hd, q_dim = sh.H * hd, kv_dim = sh.KV * hd;
+  rr.rotate = true;
   if (r < sh.H) {
-    src = a.q + (long long)token * q_dim + r * hd;
-    bias = a.b_q ? a.b_q + r * hd : nullptr;
-    w = a.q_norm;
-    dst = a.q_rot + (long long)token * q_dim + r * hd;
+    rr.src = a.q + (long long)token * q_dim + r * hd;
+    rr.bias = a.b_q ? a.b_q + r * hd : nullptr;
+    rr.w = a.q_norm;
+    rr.dst = a.q_rot + (long long)token * q_dim + r * hd;
   } else {
-    const int c = (r - sh.H) % sh.KV;
     const bool is_v = (r - sh.H) >= sh.KV;
-    const long long row = (long long)st.slot[s] * sh.seq_stride + ((long long)c * sh.cap + pos) * hd;
+    const int c = is_v ? r - sh.H - sh.KV : r - sh.H;
+    const long long row = (long long)st.slot[s] * sh.seq_stride + ((long long)c * sh.cap + rr.pos) * hd;
     if (is_v) {
-      src = a.v + (long long)token * kv_dim + c * hd;
-      bias = a.b_v ? a.b_v + c * hd : nullptr;
-      w = nullptr;
-      dst = a.vc + row;
-      rotate = false;
+      rr.src = a.v + (long long)token * kv_dim + c * hd;
+      rr.bias = a.b_v ? a.b_v + c * hd : nullptr;
+      rr.w = nullptr;
+      rr.dst = a.vc + row;
+      rr.rotate = false;
     } else {
-      src = a.k + (long long)token * kv_dim + c * hd;
-      bias = a.b_k ? a.b_k + c * hd : nullptr;
-      w = a.k_norm;
-      dst = a.kc + row;
+      rr.src = a.k + (long long)token * kv_dim + c * hd;
+      rr.bias = a.b_k ? a.b_k + c * hd : nullptr;
+      rr.w = a.k_norm;
+      rr.dst = a.kc + row;
     }
   }
+  return rr;
+}
 
-  if (!rotate) {  // V rows are stored as they are (llama_block.cr:284)
+__device__ __forceinline__ float lane_value(float x, int t) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), t));
+}
+
+// Even head_dim up to 128: R head rows per wavefront, lane i < hd/2 owns the pair
+// (i, i + hd/2).  All loads of the R rows are issued before any arithmetic.
+template <int R>
+__global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
+  const int lane = threadIdx.x & 63;
+  const int hd = sh.hd, half = hd >> 1;
+  const int token = blockIdx.y;
+  const int r0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+  const bool active = lane < half;
+  const int i = active ? lane : 0;
+  RowRef rr[R];
+  float x0[R], x1[R], w0[R], w1[R];
+  float2 cs[R];
+#pragma unroll
+  for (int u = 0; u < R; ++u) {
+    rr[u] = locate_row(a, st, sh, token, r0 + u, total_tokens);
+    x0[u] = rr[u].src[i];
+    x1[u] = rr[u].src[i + half];
+    if (rr[u].bias) {
+      x0[u] = x0[u] + rr[u].bias[i];
+      x1[u] = x1[u] + rr[u].bias[i + half];
+    }
+    w0[u] = rr[u].w ? rr[u].w[i] : 1.0f;
+    w1[u] = rr[u].w ? rr[u].w[i + half] : 1.0f;
+    cs[u] = rr[u].rotate ? a.rope_tab[(long long)rr[u].pos * half + i] : float2{1.0f, 0.0f};
+  }
+#pragma unroll
+  for (int u = 0; u < R; ++u) {
+    if (!rr[u].valid) continue;  // uniform over the wavefront
+    float *dst = rr[u].dst;
+    if (!rr[u].rotate) {  // V rows are stored as they are (llama_block.cr:284)
+      if (active) {
+        dst[i] = x0[u];
+        dst[i + half] = x1[u];
+      }
+      continue;
+    }
+    float a0 = x0[u], a1 = x1[u];
+    if (rr[u].w) {
+      // The sum of squares runs in the reference's order (d ascending, one fp32 add
+      // per element): every lane walks the row through lane broadcasts, first the
+      // lower halves of the pairs, then the upper halves.
+      float ss = 0.0f;
+      for (int t0 = 0; t0 < half; t0 += 16) {
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+          if (t0 + k < half) {
+            const float v = lane_value(a0, t0 + k);
+            const float sq = v * v;
+            ss = ss + sq;
+          }
+      }
+      for (int t0 = 0; t0 < half; t0 += 16) {
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+          if (t0 + k < half) {
+            const float v = lane_value(a1, t0 + k);
+            const float sq = v * v;
+            ss = ss + sq;
+          }
+      }
+      const float mean = ss / (float)hd;
+      const float inv = (float)(1.0 / sqrt((double)mean + a.eps));
+      a0 = a0 * inv;
+      a0 = a0 * w0[u];
+      a1 = a1 * inv;
+      a1 = a1 * w1[u];
+    }
+    if (active) {
+      const float p0 = a0 * cs[u].x, p1 = a1 * cs[u].y, p2 = a1 * cs[u].x, p3 = a0 * cs[u].y;
+      dst[i] = p0 - p1;
+      dst[i + half] = p2 + p3;
+    }
+  }
+}
+
+// Any head_dim (odd ones included): one wavefront per head row.
+__global__ __launch_bounds__(256) void prep_rows_generic_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
+  const int lane = threadIdx.x & 63;
+  const RowRef rr = locate_row(a, st, sh, blockIdx.y, blockIdx.x * 4 + (threadIdx.x >> 6), total_tokens);
+  if (!rr.valid) return;
+  const int hd = sh.hd, half = hd >> 1;
+  const float *src = rr.src, *bias = rr.bias, *w = rr.w;
+  float *dst = rr.dst;
+  const int pos = rr.pos;
+
+  if (!rr.rotate) {  // V rows are stored as they are (llama_block.cr:284)
     for (int d = lane; d < hd; d += 64) dst[d] = bias ? src[d] + bias[d] : src[d];
     return;
   }
@@ -66,8 +162,8 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st,
   float inv = 1.0f;
   if (w) {
     // The sum of squares must run in the reference's order (d ascending, one fp32
-    // add per element).  The row is fetched once, 64 elements per load, and every
-    // lane then walks it through lane broadcasts, so all lanes hold the same sum.
+    // add per element).  The row is fetched 64 elements per load, and every lane
+    // then walks it through lane broadcasts, so all lanes hold the same sum.
     float ss = 0.0f;
     for (int d0 = 0; d0 < hd; d0 += 64) {
       const int d = d0 + lane;
@@ -75,7 +171,7 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st,
       if (d < hd) x = bias ? src[d] + bias[d] : src[d];
       const int n = min(64, hd - d0);
       for (int t = 0; t < n; ++t) {
-        const float v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), t));
+        const float v = lane_value(x, t);
         const float sq = v * v;
         ss = ss + sq;
       }
@@ -119,11 +215,37 @@ __global__ void legacy_append_kernel(const float *__restrict__ staging, float *_
 hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, int total_tokens,
                        hipStream_t stream) {
   if (total_tokens <= 0) return hipSuccess;
-  const long long items = (long long)total_tokens * (sh.H + 2 * sh.KV);
-  const long long blocks = (items + 3) / 4;
-  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(prep_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, st, sh, total_tokens);
-  return hipGetLastError();
+  const int rows = sh.H + 2 * sh.KV;
+  const bool fast = sh.hd <= 128 && (sh.hd & 1) == 0;
+  // few rows (decode): one row per wavefront keeps the latency short; many rows
+  // (prefill): four rows per wavefront amortise the load latency
+  const int rows_per_wave = fast && (long long)total_tokens * rows >= 8192 ? 4 : 1;
+  const int per_wg = 4 * rows_per_wave;
+  // blockIdx.y is the token; a launch takes at most 65535 of them
+  for (int t0 = 0; t0 < total_tokens; t0 += 65535) {
+    const int nt = total_tokens - t0 < 65535 ? total_tokens - t0 : 65535;
+    PrepArgs b = a;
+    b.q += (long long)t0 * sh.H * sh.hd;
+    b.k += (long long)t0 * sh.KV * sh.hd;
+    b.v += (long long)t0 * sh.KV * sh.hd;
+    b.q_rot += (long long)t0 * sh.H * sh.hd;
+    SeqTable sub = st;
+    if (t0) {  // the kernel indexes tokens from 0: shift the prefix sums
+      for (int s = 0; s <= st.n_seqs; ++s) sub.tok_off[s] = st.tok_off[s] - t0;
+    }
+    dim3 grid((unsigned)((rows + per_wg - 1) / per_wg), (unsigned)nt);
+    // n_seqs == tokens means one row per sequence (decode) only for the whole call
+    const int tt = t0 == 0 && nt == total_tokens ? total_tokens : -1;
+    if (!fast)
+      hipLaunchKernelGGL(prep_rows_generic_kernel, grid, dim3(256), 0, stream, b, sub, sh, tt);
+    else if (rows_per_wave == 4)
+      hipLaunchKernelGGL(prep_rows_kernel<4>, grid, dim3(256), 0, stream, b, sub, sh, tt);
+    else
+      hipLaunchKernelGGL(prep_rows_kernel<1>, grid, dim3(256), 0, stream, b, sub, sh, tt);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
