@@ -57,9 +57,17 @@ struct DecodePlan {
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 
-hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
-                         const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
-                         hipStream_t stream, hipEvent_t before_split = nullptr, hipEvent_t after_split = nullptr);
+// q_rot: rotated queries [rows][H*hd]; the cache already holds the new rows.
+// pair_count: one zero-initialised int per (sequence, kv head); the kernel leaves it zero.
+struct DecodeArgs {
+  const float *q_rot;
+  const float *kc, *vc;
+  float *out;
+  float *partials;
+  int *pair_count;
+};
+hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
+                         hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr);
 // wgs_per_cu: 0 = default; 1..3 pads the kernel's LDS so that at most that many
 // workgroups share a compute unit (a tuning knob).
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,

@@ -78,6 +78,8 @@ struct shainet_attn_ctx {
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
+  int *pair_count = nullptr;
+  size_t pair_count_cap = 0;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
@@ -148,10 +150,31 @@ Shape shape_of(const shainet_attn_ctx *c, int cap) {
   return sh;
 }
 
-// Attention of already rotated rows over a cache: shared by the fused entry
-// point and by attention_kv_f32.
-int run_attention(shainet_attn_ctx *c, const float *q_rot, const float *kc, const float *vc, float *out,
-                  SeqTable &st, const Shape &sh, int total_tokens, float scale, hipStream_t stream) {
+// Zero-initialised ints, one per (sequence, kv head), for the decode kernel's
+// last-arriver merge.  The kernel leaves them zero.
+int ensure_pair_counters(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
+  if (n <= c->pair_count_cap) return SHAINET_HIP_OK;
+  size_t want = c->pair_count_cap ? c->pair_count_cap : 256;
+  while (want < n) want *= 2;
+  int *np = nullptr;
+  HIP_TRY(hipMalloc((void **)&np, want * sizeof(int)));
+  hipError_t e = hipMemsetAsync(np, 0, want * sizeof(int), stream);
+  if (e != hipSuccess) {
+    (void)hipFree(np);
+    return hip_fail(e, "hipMemsetAsync(pair counters)");
+  }
+  if (c->pair_count) (void)hipFree(c->pair_count);  // hipFree waits for the device
+  c->pair_count = np;
+  c->pair_count_cap = want;
+  return SHAINET_HIP_OK;
+}
+
+// Attention over a cache: shared by the fused entry point and by attention_kv_f32.
+// prep != nullptr: the rows are raw projection outputs; the prep kernel does bias,
+// QK-norm, RoPE and the append first.  prep == nullptr: q_rot holds rotated
+// queries and the cache already holds the new rows.
+int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc, float *out, SeqTable &st,
+                  const Shape &sh, int total_tokens, float scale, hipStream_t stream, const PrepArgs *prep) {
   const Path path = choose_path(st, sh);
   hipError_t e;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -164,18 +187,36 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, const float *kc, cons
   if (path == Path::kDecodeSplitK) {
     const DecodePlan plan = plan_decode(st, sh, c->decode_wgs_override);
     int rc = c->partials.reserve(decode_partial_floats(sh, plan));
+    if (!rc) rc = ensure_pair_counters(c, (size_t)st.n_seqs * sh.KV, stream);
     if (rc) return rc;
-    e = launch_decode(q_rot, kc, vc, out, c->partials.p, st, sh, plan, scale, stream, ev0, ev1);
-  } else if (path == Path::kPrefillMfma) {
-    const int items = plan_work(st, sh, path);
-    if (ev0) (void)hipEventRecord(ev0, stream);
-    e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream, c->prefill_wgs_per_cu);
-    if (ev1) (void)hipEventRecord(ev1, stream);
+    DecodeArgs d;
+    d.q_rot = q_rot;
+    d.kc = kc;
+    d.vc = vc;
+    d.out = out;
+    d.partials = c->partials.p;
+    d.pair_count = c->pair_count;
+    if (prep) {
+      e = launch_prep(*prep, st, sh, total_tokens, stream);
+      if (e != hipSuccess) return hip_fail(e, "prep launch");
+    }
+    e = launch_decode(d, st, sh, plan, scale, stream, ev0, ev1);
   } else {
-    plan_work(st, sh, path);
-    if (ev0) (void)hipEventRecord(ev0, stream);
-    e = launch_generic(q_rot, kc, vc, out, st, sh, total_tokens, scale, stream);
-    if (ev1) (void)hipEventRecord(ev1, stream);
+    if (prep) {
+      e = launch_prep(*prep, st, sh, total_tokens, stream);
+      if (e != hipSuccess) return hip_fail(e, "prep launch");
+    }
+    if (path == Path::kPrefillMfma) {
+      const int items = plan_work(st, sh, path);
+      if (ev0) (void)hipEventRecord(ev0, stream);
+      e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream, c->prefill_wgs_per_cu);
+      if (ev1) (void)hipEventRecord(ev1, stream);
+    } else {
+      plan_work(st, sh, path);
+      if (ev0) (void)hipEventRecord(ev0, stream);
+      e = launch_generic(q_rot, kc, vc, out, st, sh, total_tokens, scale, stream);
+      if (ev1) (void)hipEventRecord(ev1, stream);
+    }
   }
   if (e != hipSuccess) return hip_fail(e, "attention launch");
   return SHAINET_HIP_OK;
@@ -237,7 +278,9 @@ void attention_kv_f32(const float *q, const float *kc, const float *vc, float *o
   st.n_new[0] = new_tokens;
   st.tok_off[1] = new_tokens;
   Shape sh = shape_of(c, capacity);
-  int rc = run_attention(c, q, kc, vc, out, st, sh, new_tokens, scale, nullptr);
+  // the cache is only read on this path
+  int rc = run_attention(c, q, const_cast<float *>(kc), const_cast<float *>(vc), out, st, sh, new_tokens, scale,
+                         nullptr, nullptr);
   if (rc) fprintf(stderr, "HIP Error in attention_kv_f32: %s\n", g_err);
 }
 
@@ -313,6 +356,7 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
   for (float *p : {c->d_q_norm, c->d_k_norm, c->d_bq, c->d_bk, c->d_bv})
     if (p) (void)hipFree(p);
   if (c->d_rope) (void)hipFree(c->d_rope);
+  if (c->pair_count) (void)hipFree(c->pair_count);
   for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
   delete c;
@@ -532,12 +576,10 @@ int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *s
   pa.q_rot = c->q_rot.p;
   pa.kc = kc->k;
   pa.vc = kc->v;
-  hipError_t e = launch_prep(pa, st, sh, rows, c->stream);
-  if (e != hipSuccess) return hip_fail(e, "prep launch");
-  // the rows are in the cache from here on: @cache_len = total_len (llama_block.cr:288-289)
+  // the rows are in the cache once this call's kernels have run: @cache_len = total_len (llama_block.cr:288-289)
   for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
   c->last_rows = rows;
-  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream);
+  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa);
   if (rc) return rc;
   if (mem == SHAINET_HIP_MEM_HOST) {
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));

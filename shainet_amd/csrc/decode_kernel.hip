@@ -10,8 +10,9 @@
 // sequence lengths are.  A span that crosses a pair boundary is processed as two
 // segments.  The four wavefronts of a workgroup take the tiles of a segment
 // round-robin, each keeping its own online softmax, and merge through LDS into
-// one partial (max, sum, O) per segment; a second kernel merges the partials of
-// each pair.
+// one partial (max, sum, O) per segment; the workgroup that delivers the last
+// partial of a pair (an atomic counter per pair tells) merges them and writes the
+// output row, so a decode step is one launch.
 //
 // Per 16-key tile a wavefront
 //   * copies the K tile (16 contiguous rows) from HBM straight into LDS with
@@ -44,6 +45,18 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Split-K partials cross workgroups that may sit on different XCDs, whose L2
+// caches are not kept coherent with each other for ordinary accesses.  Relaxed
+// atomic accesses at agent scope compile to write-through stores and cache-
+// bypassing loads, which is all that is needed for data published through an
+// atomic counter.
+__device__ __forceinline__ void coherent_store(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(uintptr_t)(p))
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
@@ -87,15 +100,15 @@ template <int HD>
 __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__restrict__ q_rot,
                                                                const float *__restrict__ kc,
                                                                const float *__restrict__ vc,
-                                                               float *__restrict__ out,
-                                                               float *__restrict__ part_o,
-                                                               float *__restrict__ part_ml, SeqTable st,
+                                                               float *__restrict__ out, float *part_o,
+                                                               float *part_ml, int *pair_count, SeqTable st,
                                                                Shape sh, int tiles_per_wg, int total_tiles,
                                                                int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   __shared__ __attribute__((aligned(1024))) char k_lds[4][2][C::TILE_BYTES];
   extern __shared__ float merge_lds[];  // [4][g][HD] O, [4][g] max, [4][g] sum
+  __shared__ bool last_flag;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, j = lane >> 4;
@@ -119,7 +132,18 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
     const float *vbase = vc + head_base;
     const int token = st.tok_off[s];
 
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    f32x4 v_next[4][C::NVU];
+    int tile = tile0 + wave;
     float qr[HD / 4];
+    if (tile < tile1) {
+      issue_k_tile<HD>(kbase, tile * 16, L - 1, my_lds, lane);
+      load_v_tile<HD>(vbase, tile * 16, L - 1, col, j, v_next);
+    }
     {
       const float *qp = q_rot + ((long long)token * sh.H + kvh * g + (col < g ? col : 0)) * HD + 4 * j;
 #pragma unroll
@@ -131,18 +155,6 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         qr[4 * i + 2] = x.z;
         qr[4 * i + 3] = x.w;
       }
-    }
-
-    float m = -INFINITY, l = 0.f;
-    f32x4 o[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    f32x4 v_next[4][C::NVU];
-    int tile = tile0 + wave;
-    if (tile < tile1) {
-      issue_k_tile<HD>(kbase, tile * 16, L - 1, my_lds, lane);
-      load_v_tile<HD>(vbase, tile * 16, L - 1, col, j, v_next);
     }
     for (int it = 0; tile < tile1; tile += 4, ++it) {
       const int kb = tile * 16;
@@ -236,65 +248,79 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         out[((long long)token * sh.H + kvh * g + cc) * HD + d] = acc / ls;
       } else if (slot < n_slots) {
         const long long pi = (long long)slot * g + cc;
-        part_o[pi * HD + d] = acc;
+        coherent_store(&part_o[pi * HD + d], acc);
         if (d == 0) {
-          part_ml[2 * pi] = mm;
-          part_ml[2 * pi + 1] = ls;
+          coherent_store(&part_ml[2 * pi], mm);
+          coherent_store(&part_ml[2 * pi + 1], ls);
+        }
+      }
+    }
+    if (!whole_pair) {
+      // The last workgroup to deliver a partial of this pair merges them all.  The
+      // counter returns to zero for the next launch.
+      const int a = st.work_off[s] + kvh * n_s;  // the pair's tiles are [a, a + n_s)
+      const int w_lo = a / tiles_per_wg, w_hi = (a + n_s - 1) / tiles_per_wg;
+      const int n_part = w_hi - w_lo + 1;
+      // Partials are written through to device-coherent memory (coherent_store);
+      // the barrier waits for this workgroup's stores to be acknowledged before
+      // its arrival is counted.
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        const int old = atomicAdd(&pair_count[pair], 1);
+        last_flag = old == n_part - 1;
+        if (last_flag) atomicExch(&pair_count[pair], 0);
+      }
+      __syncthreads();
+      if (last_flag) {
+        // every partial of the pair is in memory: drop whatever this XCD's caches
+        // still hold of those addresses, then read them with ordinary wide loads
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        constexpr int LPR = HD / 4;       // lanes that cover one row with float4
+        constexpr int GROUPS = 64 / LPR;  // partials handled side by side
+        const int d4 = lane % LPR, grp = lane / LPR;
+        const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
+        for (int cc = wave; cc < g; cc += 4) {
+          const long long first = base + cc;
+          float mm = -INFINITY;
+          for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
+          for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
+          float ls = 0.f;
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+          for (int i0 = 0; i0 < n_part; i0 += 8 * GROUPS) {  // eight rows in flight per lane
+            f32x4 x[8];
+            float f[8], lp[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int i = i0 + u * GROUPS + grp;
+              const long long pi = first + (long long)min(i, n_part - 1) * g;
+              x[u] = *(const f32x4 *)&part_o[pi * HD + 4 * d4];
+              f[u] = part_ml[2 * pi];
+              lp[u] = part_ml[2 * pi + 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int i = i0 + u * GROUPS + grp;
+              const float w = i < n_part ? fast_exp2((f[u] - mm) * c) : 0.f;
+              acc += w * x[u];
+              ls += w * lp[u];
+            }
+          }
+#pragma unroll
+          for (int o2 = LPR; o2 < 64; o2 <<= 1) {
+            acc.x += __shfl_xor(acc.x, o2);
+            acc.y += __shfl_xor(acc.y, o2);
+            acc.z += __shfl_xor(acc.z, o2);
+            acc.w += __shfl_xor(acc.w, o2);
+            ls += __shfl_xor(ls, o2);
+          }
+          if (grp == 0) {
+            const float inv = 1.0f / ls;
+            *(f32x4 *)&out[((long long)token * sh.H + kvh * g + cc) * HD + 4 * d4] = acc * inv;
+          }
         }
       }
     }
     t += seg_tiles;
-  }
-}
-
-// Merge the partials of one (sequence, head): one wavefront each.
-__global__ __launch_bounds__(256) void decode_combine_kernel(const float *__restrict__ part_o,
-                                                             const float *__restrict__ part_ml,
-                                                             float *__restrict__ out, SeqTable st, Shape sh,
-                                                             int tiles_per_wg, float c) {
-  const int lane = threadIdx.x & 63;
-  const int id = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (id >= st.n_seqs * sh.H) return;
-  const int s = id / sh.H, h = id - s * sh.H;
-  const int kvh = h / sh.g, cc = h - kvh * sh.g;
-  const int n_s = (st.start_pos[s] + 1 + 15) >> 4;
-  const int a = st.work_off[s] + kvh * n_s;  // the pair's tiles are [a, a + n_s)
-  const int w_lo = a / tiles_per_wg, w_hi = (a + n_s - 1) / tiles_per_wg;
-  if (w_lo == w_hi) return;  // one workgroup held the whole pair and wrote the output itself
-  const int pair = s * sh.KV + kvh;
-  const int n = w_hi - w_lo + 1;
-  const int hd = sh.hd;
-  const long long first = (long long)(w_lo + pair) * sh.g + cc;  // partial of workgroup w is first + (w - w_lo)*g
-
-  float mm = -INFINITY;
-  for (int i = lane; i < n; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * sh.g)]);
-  for (int o = 32; o > 0; o >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o));
-  float ls = 0.f;
-  for (int i = lane; i < n; i += 64) {
-    const long long pi = first + (long long)i * sh.g;
-    ls += fast_exp2((part_ml[2 * pi] - mm) * c) * part_ml[2 * pi + 1];
-  }
-  for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
-  const float inv = 1.0f / ls;
-  for (int d = lane; d < hd; d += 64) {
-    float acc = 0.f;
-    int i = 0;
-    for (; i + 4 <= n; i += 4) {  // four independent loads in flight
-      float f[4], x[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const long long pi = first + (long long)(i + u) * sh.g;
-        f[u] = part_ml[2 * pi];
-        x[u] = part_o[pi * hd + d];
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) acc += fast_exp2((f[u] - mm) * c) * x[u];
-    }
-    for (; i < n; ++i) {
-      const long long pi = first + (long long)i * sh.g;
-      acc += fast_exp2((part_ml[2 * pi] - mm) * c) * part_o[pi * hd + d];
-    }
-    out[((long long)st.tok_off[s] * sh.H + h) * hd + d] = acc * inv;
   }
 }
 
@@ -322,33 +348,30 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
   return (size_t)p.n_slots * sh.g * (sh.hd + 2);
 }
 
-hipError_t launch_decode(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
-                         const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
-                         hipStream_t stream, hipEvent_t before_split, hipEvent_t after_split) {
+hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
+                         hipStream_t stream, hipEvent_t before, hipEvent_t after) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
-      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1)
+      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.pair_count)
     return hipErrorInvalidValue;
   for (int s = 0; s < st.n_seqs; ++s)
     if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
       return hipErrorInvalidValue;
-  float *part_o = partials;
-  float *part_ml = partials + (size_t)p.n_slots * sh.g * sh.hd;
+  if (!d.q_rot) return hipErrorInvalidValue;
+  float *part_o = d.partials;
+  float *part_ml = d.partials + (size_t)p.n_slots * sh.g * sh.hd;
   const float c = scale * kLog2e;
   const size_t smem = (size_t)(4 * sh.g * sh.hd + 8 * sh.g) * sizeof(float);
-  if (before_split) (void)hipEventRecord(before_split, stream);
+  if (before) (void)hipEventRecord(before, stream);
+  dim3 grid((unsigned)p.n_wgs), block(256);
   if (sh.hd == 64)
-    hipLaunchKernelGGL(decode_splitk_kernel<64>, dim3((unsigned)p.n_wgs), dim3(256), smem, stream, q_rot, kc, vc,
-                       out, part_o, part_ml, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipLaunchKernelGGL(decode_splitk_kernel<64>, grid, block, smem, stream, d.q_rot, d.kc, d.vc, d.out, part_o,
+                       part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
   else
-    hipLaunchKernelGGL(decode_splitk_kernel<128>, dim3((unsigned)p.n_wgs), dim3(256), smem, stream, q_rot, kc, vc,
-                       out, part_o, part_ml, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipLaunchKernelGGL(decode_splitk_kernel<128>, grid, block, smem, stream, d.q_rot, d.kc, d.vc, d.out, part_o,
+                       part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
   hipError_t e = hipGetLastError();
-  if (after_split) (void)hipEventRecord(after_split, stream);
-  if (e != hipSuccess) return e;
-  const int waves = st.n_seqs * sh.H;
-  hipLaunchKernelGGL(decode_combine_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, part_o,
-                     part_ml, out, st, sh, p.tiles_per_wg, c);
-  return hipGetLastError();
+  if (after) (void)hipEventRecord(after, stream);
+  return e;
 }
 
 }  // namespace shainet

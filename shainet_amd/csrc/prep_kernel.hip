@@ -11,6 +11,7 @@
 //     (275-277), and x0*c - x1*s, x1*c + x0*s are separately rounded (280-281).
 // This file is compiled with -ffp-contract=off: no product may fuse into an add.
 #include "attn_kernels.hpp"
+#include "prep_math.hpp"
 
 #pragma clang fp contract(off)
 
@@ -64,10 +65,6 @@ __device__ __forceinline__ RowRef locate_row(const PrepArgs &a, const SeqTable &
   return rr;
 }
 
-__device__ __forceinline__ float lane_value(float x, int t) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), t));
-}
-
 // Even head_dim up to 128: R head rows per wavefront, lane i < hd/2 owns the pair
 // (i, i + hd/2).  All loads of the R rows are issued before any arithmetic.
 template <int R>
@@ -105,41 +102,11 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st,
       }
       continue;
     }
-    float a0 = x0[u], a1 = x1[u];
-    if (rr[u].w) {
-      // The sum of squares runs in the reference's order (d ascending, one fp32 add
-      // per element): every lane walks the row through lane broadcasts, first the
-      // lower halves of the pairs, then the upper halves.
-      float ss = 0.0f;
-      for (int t0 = 0; t0 < half; t0 += 16) {
-#pragma unroll
-        for (int k = 0; k < 16; ++k)
-          if (t0 + k < half) {
-            const float v = lane_value(a0, t0 + k);
-            const float sq = v * v;
-            ss = ss + sq;
-          }
-      }
-      for (int t0 = 0; t0 < half; t0 += 16) {
-#pragma unroll
-        for (int k = 0; k < 16; ++k)
-          if (t0 + k < half) {
-            const float v = lane_value(a1, t0 + k);
-            const float sq = v * v;
-            ss = ss + sq;
-          }
-      }
-      const float mean = ss / (float)hd;
-      const float inv = (float)(1.0 / sqrt((double)mean + a.eps));
-      a0 = a0 * inv;
-      a0 = a0 * w0[u];
-      a1 = a1 * inv;
-      a1 = a1 * w1[u];
-    }
+    float y0, y1;
+    norm_rotate_pair(x0[u], x1[u], rr[u].w != nullptr, w0[u], w1[u], a.eps, hd, half, cs[u], y0, y1);
     if (active) {
-      const float p0 = a0 * cs[u].x, p1 = a1 * cs[u].y, p2 = a1 * cs[u].x, p3 = a0 * cs[u].y;
-      dst[i] = p0 - p1;
-      dst[i + half] = p2 + p3;
+      dst[i] = y0;
+      dst[i + half] = y1;
     }
   }
 }
