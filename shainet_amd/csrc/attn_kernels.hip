@@ -45,28 +45,13 @@ __device__ __forceinline__ int find_seq(const SeqTable &st, int item, const int 
 //            j = l/32 covers d = 8*(s/4) + 4*j + s%4 (float4 pieces of a K row).
 //   output:  tile t, m = d index (d = NT*m + t), contraction over the tile's keys in
 //            the order the score accumulator holds them.
-template <int HD>
-__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__restrict__ q_rot,
-                                                              const float *__restrict__ kc,
-                                                              const float *__restrict__ vc,
-                                                              float *__restrict__ out, SeqTable st, Shape sh,
-                                                              float c) {
-  constexpr int NK4 = HD / 8;   // float4 pieces of a K row per lane
-  constexpr int NT = HD / 32;   // d tiles of the output
-  constexpr int KSTR = HD + 4;  // padded K row stride in LDS: conflict-free 16-byte reads down a column
-  constexpr int LD4 = HD / 32;  // float4 per thread to stage one K (or V) tile
-  __shared__ float Ks[2][32 * KSTR];
-  __shared__ float Vs[2][32 * HD];
-
-  // Workgroups are numbered so that the hardware dispatcher, which hands them out in
-  // index order, starts the row blocks with the longest key ranges first: level 0
-  // is every sequence's last block, level 1 the one before, and so on; the kv head
-  // is the fastest index, so with 8 kv heads each XCD (index % 8) keeps to one head
-  // and its K/V stay in that XCD's L2.  st.work_off[s] = row blocks of sequence s,
-  // st.ord = sequences by descending block count.
-  const int kvh = blockIdx.x % sh.KV;
-  int rank = blockIdx.x / sh.KV;
-  int s = 0, level = 0;
+// Row block number `rank` in dispatch order -> (sequence, block).  Level 0 is every
+// sequence's last block (the longest key range), level 1 the one before, and so
+// on.  st.work_off[s] = row blocks of sequence s, st.ord = sequences by descending
+// block count.
+__device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &s, int &vb) {
+  s = 0;
+  int level = 0;
   for (int b = st.n_seqs - 1; b >= 0; --b) {  // levels [n_{b+1}, n_b) have b+1 active sequences
     const int lo = b + 1 < st.n_seqs ? st.work_off[st.ord[b + 1]] : 0;
     const int cnt = (st.work_off[st.ord[b]] - lo) * (b + 1);
@@ -77,7 +62,35 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
     }
     rank -= cnt;
   }
-  const int vb = st.work_off[s] - 1 - level;
+  vb = st.work_off[s] - 1 - level;
+}
+
+template <int HD>
+__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__restrict__ q_rot,
+                                                              const float *__restrict__ kc,
+                                                              const float *__restrict__ vc,
+                                                              float *__restrict__ out,
+                                                              float *__restrict__ part_o,
+                                                              float *__restrict__ part_ml, SeqTable st,
+                                                              Shape sh, int ns, float c) {
+  constexpr int NK4 = HD / 8;   // float4 pieces of a K row per lane
+  constexpr int NT = HD / 32;   // d tiles of the output
+  constexpr int KSTR = HD + 4;  // padded K row stride in LDS: conflict-free 16-byte reads down a column
+  constexpr int LD4 = HD / 32;  // float4 per thread to stage one K (or V) tile
+  __shared__ float Ks[2][32 * KSTR];
+  __shared__ float Vs[2][32 * HD];
+
+  // Workgroups are numbered so that the hardware dispatcher, which hands them out in
+  // index order, starts the row blocks with the longest key ranges first; the kv
+  // head is the fastest index, so with 8 kv heads each XCD (index % 8) keeps to one
+  // head and its K/V stay in that XCD's L2.  When a launch has too few row blocks to
+  // fill the chip, each block's key range is cut into ns chunks that run as separate
+  // workgroups and leave partial (max, sum, O) rows for prefill_combine_kernel.
+  const int kvh = blockIdx.x % sh.KV;
+  const int chunk = (blockIdx.x / sh.KV) % ns;
+  const int item = blockIdx.x / sh.KV / ns;
+  int s, vb;
+  locate_block(st, item, s, vb);
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
   const int L = S + T, VR = T * g;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -93,6 +106,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   const int wave_hi = wave_active ? S + min(v0 + 31, VR - 1) / g : -1;  // largest
   const int wg_hi = S + min(vb * 128 + 127, VR - 1) / g;
   const int n_tiles = wg_hi / 32 + 1;
+  const int tiles_per_chunk = (n_tiles + ns - 1) / ns;
+  const int kt0 = chunk * tiles_per_chunk, kt1 = min(n_tiles, kt0 + tiles_per_chunk);
   const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
   const float *kbase = kc + head_base;
   const float *vbase = vc + head_base;
@@ -140,13 +155,15 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
     }
   };
 
-  load_tile(0);
-  store_tile(0);
+  if (kt0 < kt1) {
+    load_tile(kt0);
+    store_tile(kt0 & 1);
+  }
   __syncthreads();
 
-  for (int kt = 0; kt < n_tiles; ++kt) {
+  for (int kt = kt0; kt < kt1; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < n_tiles) load_tile(kt + 1);
+    if (kt + 1 < kt1) load_tile(kt + 1);
     if (kt * 32 <= wave_hi) {
       f32x16 sacc;
 #pragma unroll
@@ -171,9 +188,11 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float mnew = fmaxf(m, mx);  // finite from tile 0 on: key 0 is visible to every row
-      const float alpha = fast_exp2((m - mnew) * c);
-      const float mc = mnew * c;
+      const float mnew = fmaxf(m, mx);
+      // a chunk that starts past a row's last visible key leaves that row at -inf
+      const float mref = mnew == -INFINITY ? 0.f : mnew;
+      const float alpha = fast_exp2((m - mref) * c);
+      const float mc = mref * c;
       float psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -205,12 +224,25 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
         }
       }
     }
-    if (kt + 1 < n_tiles) store_tile(buf ^ 1);
+    if (kt + 1 < kt1) store_tile(buf ^ 1);
     __syncthreads();
   }
 
   l += __shfl_xor(l, 32);
-  if (valid) {
+  if (ns > 1) {  // unnormalised partial of this key chunk: [128 virtual rows][HD], (max, sum) per row
+    const long long pbase = (((long long)item * sh.KV + kvh) * ns + chunk) * 128 + wave * 32 + n;
+    float *op = part_o + pbase * HD;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int d = NT * (8 * (r >> 2) + 4 * j + (r & 3));
+      if constexpr (NT == 2) {
+        *(float2 *)(op + d) = float2{o[0][r], o[1][r]};
+      } else {
+        *(f32x4 *)(op + d) = f32x4{o[0][r], o[1][r], o[2][r], o[3][r]};
+      }
+    }
+    if (j == 0) *(float2 *)(part_ml + 2 * pbase) = float2{m, l};
+  } else if (valid) {
     const float inv = 1.0f / l;
     float *op = out + qo_off;
 #pragma unroll
@@ -222,6 +254,36 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
         *(f32x4 *)(op + d) = f32x4{o[0][r] * inv, o[1][r] * inv, o[2][r] * inv, o[3][r] * inv};
       }
     }
+  }
+}
+
+// Merge the key chunks of one (row block, kv head): online-softmax combine per row.
+__global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ part_o,
+                                                              const float *__restrict__ part_ml,
+                                                              float *__restrict__ out, SeqTable st, Shape sh,
+                                                              int ns, float c) {
+  const int kvh = blockIdx.x % sh.KV, item = blockIdx.x / sh.KV;
+  int s, vb;
+  locate_block(st, item, s, vb);
+  const int g = sh.g, hd = sh.hd, hd4 = hd >> 2;
+  const int VR = st.n_new[s] * g;
+  const long long base = ((long long)item * sh.KV + kvh) * ns * 128;
+  for (int idx = threadIdx.x; idx < 128 * hd4; idx += 256) {
+    const int vl = idx / hd4, d4 = idx - vl * hd4;
+    const int v = vb * 128 + vl;
+    if (v >= VR) continue;
+    const int row = v / g, hg = v - row * g;
+    float mm = -INFINITY;
+    for (int k = 0; k < ns; ++k) mm = fmaxf(mm, part_ml[2 * (base + (long long)k * 128 + vl)]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float ls = 0.f;
+    for (int k = 0; k < ns; ++k) {
+      const long long pi = base + (long long)k * 128 + vl;
+      const float f = fast_exp2((part_ml[2 * pi] - mm) * c);  // 0 for a chunk that saw no visible key
+      acc += f * *(const f32x4 *)(part_o + pi * hd + 4 * d4);
+      ls += f * part_ml[2 * pi + 1];
+    }
+    *(f32x4 *)(out + ((long long)(st.tok_off[s] + row) * sh.H + kvh * g + hg) * hd + 4 * d4) = acc * (1.0f / ls);
   }
 }
 
@@ -331,29 +393,58 @@ static bool table_ok(const SeqTable &st, const Shape &sh) {
   return true;
 }
 
-hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
-                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream,
-                          int wgs_per_cu) {
-  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1) return hipErrorInvalidValue;
-  if ((long long)items * sh.KV > 0x7fffffffLL) return hipErrorInvalidValue;
+int prefill_key_splits(const SeqTable &st, const Shape &sh, int items) {
+  const long long wgs = (long long)items * sh.KV;
+  if (wgs >= 384) return 1;
+  int longest = 0;  // key tiles of the longest row block
+  for (int s = 0; s < st.n_seqs; ++s) {
+    const int t = (st.start_pos[s] + st.n_new[s] + 31) / 32;
+    longest = t > longest ? t : longest;
+  }
+  int ns = (int)((512 + wgs - 1) / wgs);
+  const int cap = longest / 8;  // at least eight key tiles per chunk
+  if (ns > cap) ns = cap;
+  if (ns > 16) ns = 16;
+  return ns < 1 ? 1 : ns;
+}
+
+size_t prefill_partial_floats(const Shape &sh, int items, int ns) {
+  return ns > 1 ? (size_t)items * sh.KV * ns * 128 * (sh.hd + 2) : 0;
+}
+
+hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
+                          const SeqTable &st, const Shape &sh, int items, int ns, float scale,
+                          hipStream_t stream, int wgs_per_cu) {
+  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1 || ns < 1 || (ns > 1 && !partials))
+    return hipErrorInvalidValue;
+  const long long n_wgs = (long long)items * sh.KV * ns;
+  if (n_wgs > 0x7fffffffLL) return hipErrorInvalidValue;
   const float c = scale * kLog2e;
-  dim3 grid((unsigned)(items * sh.KV));
+  dim3 grid((unsigned)n_wgs);
+  float *part_o = partials;
+  float *part_ml = partials ? partials + (size_t)items * sh.KV * ns * 128 * sh.hd : nullptr;
   // static LDS of the kernel: two stages of a padded K tile and a V tile
   const size_t static_lds = (size_t)2 * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
   size_t pad = 0;
   // With fewer workgroups than three per compute unit everything is resident at
   // once and the dispatcher cannot balance the triangular work: one workgroup per
   // compute unit lets it hand the short row blocks to whichever unit finishes first.
-  if (wgs_per_cu == 0 && (long long)items * sh.KV <= 768) wgs_per_cu = 1;
+  if (wgs_per_cu == 0 && n_wgs <= 768) wgs_per_cu = 1;
   if (wgs_per_cu >= 1 && wgs_per_cu <= 3) {
     const size_t want = (size_t)160 * 1024 / wgs_per_cu;  // one more workgroup would not fit
     const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
     if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
   }
   if (sh.hd == 64)
-    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, st, sh, c);
+    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, part_ml,
+                       st, sh, ns, c);
   else
-    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, st, sh, c);
+    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, part_ml,
+                       st, sh, ns, c);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || ns == 1) return e;
+  hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV)), dim3(256), 0, stream, part_o, part_ml,
+                     out, st, sh, ns, c);
   return hipGetLastError();
 }
 

@@ -68,11 +68,16 @@ struct DecodeArgs {
 };
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr);
+// Key splits of a prefill launch: 1 when the row blocks alone fill the chip, more
+// when they do not (few new rows on a long cached prefix); each split leaves
+// partial rows in `partials` (prefill_partial_floats) and a second kernel merges.
+int prefill_key_splits(const SeqTable &st, const Shape &sh, int items);
+size_t prefill_partial_floats(const Shape &sh, int items, int ns);
 // wgs_per_cu: 0 = default; 1..3 pads the kernel's LDS so that at most that many
 // workgroups share a compute unit (a tuning knob).
-hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out,
-                          const SeqTable &st, const Shape &sh, int items, float scale, hipStream_t stream,
-                          int wgs_per_cu = 0);
+hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
+                          const SeqTable &st, const Shape &sh, int items, int ns, float scale,
+                          hipStream_t stream, int wgs_per_cu = 0);
 hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);

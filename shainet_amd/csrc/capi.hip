@@ -83,6 +83,7 @@ struct shainet_attn_ctx {
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
+  int prefill_splits_override = 0;  // 0 = default number of key splits of the prefill kernel
   bool profiling = false;
   std::vector<hipEvent_t> prof_events;  // start, stop, start, stop, ...
 };
@@ -208,8 +209,12 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     }
     if (path == Path::kPrefillMfma) {
       const int items = plan_work(st, sh, path);
+      int ns = c->prefill_splits_override > 0 ? c->prefill_splits_override : prefill_key_splits(st, sh, items);
+      int rc = c->partials.reserve(prefill_partial_floats(sh, items, ns));
+      if (rc) return rc;
       if (ev0) (void)hipEventRecord(ev0, stream);
-      e = launch_prefill(q_rot, kc, vc, out, st, sh, items, scale, stream, c->prefill_wgs_per_cu);
+      e = launch_prefill(q_rot, kc, vc, out, c->partials.p, st, sh, items, ns, scale, stream,
+                         c->prefill_wgs_per_cu);
       if (ev1) (void)hipEventRecord(ev1, stream);
     } else {
       plan_work(st, sh, path);
@@ -314,6 +319,7 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
     if (v >= 1 && v <= 65536) c->decode_wgs_override = v;
   }
   if (const char *env = getenv("SHAINET_HIP_PREFILL_WGS_PER_CU")) c->prefill_wgs_per_cu = atoi(env);
+  if (const char *env = getenv("SHAINET_HIP_PREFILL_SPLITS")) c->prefill_splits_override = atoi(env);
   int rc = SHAINET_HIP_OK;
   hipError_t e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
   if (e != hipSuccess) rc = hip_fail(e, "hipStreamCreate");

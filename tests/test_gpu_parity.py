@@ -251,6 +251,19 @@ def test_prefill_small_shapes(hip, H, KV, hd, S, T, norm):
     check_cache_bits(cache, blocks)
 
 
+@pytest.mark.parametrize("ns", [2, 3, 5])
+def test_prefill_key_splits(hip, ns, monkeypatch):
+    # key range of every row block cut into ns chunks merged by a second kernel; with S = 0 the later
+    # chunks start past the last visible key of the early rows (their partial stays at -inf)
+    monkeypatch.setenv("SHAINET_HIP_PREFILL_SPLITS", str(ns))
+    for H, KV, hd, S, T, norm in [(8, 2, 64, 0, 70, False), (8, 1, 128, 100, 37, True), (6, 2, 64, 300, 130, False)]:
+        ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=norm, capacity=512, seed=ns + T)
+        if S:
+            check_step(ctx, cache, blocks, r, [S])
+        check_step(ctx, cache, blocks, r, [T], what=f"ns={ns} hd={hd} S={S} T={T}")
+        check_step(ctx, cache, blocks, r, [3])
+
+
 def test_prefill_then_decode_equals_one_prefill(hip):
     # chunking invariance: T rows at once == in chunks == row by row (to fp32 round-off)
     H, KV, hd, T = 8, 2, 64, 97
