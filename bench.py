@@ -11,7 +11,7 @@ fp32, batch 16 with cached lengths drawn uniform in [2048, 8192].  The other
 configurations are timed as well and reported under "workloads".
 
 Prints ONE JSON line.  `value` is microseconds per layer-step of the headline
-workload (whole step: prep + split-K + combine kernels); `roofline` prices the
+workload (whole step: the prep kernel and the split-K decode kernel); `roofline` prices the
 split-K decode kernel against HBM, `roofline_prefill` the MFMA prefill kernel
 against the fp32 matrix peak; `cpu_baseline` times the CPU oracle (a C
 restatement of the reference's single-threaded Crystal path) on the host cores.
@@ -178,6 +178,28 @@ def cpu_baseline(w, reps):
     return times[len(times) // 2] * 1e6
 
 
+def layer_decode(sa, np, steps):
+    """BASELINE configs[0] on the device: one Llama-3.2-1B-shaped attention layer (hidden 2048, 32 Q /
+    8 KV heads, head_dim 64), projections included, 512 cached positions, one new row per call, host
+    pointers in and out (so the time includes the PCIe copies and the synchronisation)."""
+    r = np.random.default_rng(1)
+    d, H, KV, hd = 2048, 32, 8, 64
+    blk = sa.LlamaBlock(d, H, rope_theta=5e5, num_kv_heads=KV)
+    blk.set_weights(*[(0.02 * r.standard_normal(sh)).astype(np.float32)
+                      for sh in ((d, H * hd), (d, KV * hd), (d, KV * hd), (H * hd, d))])
+    blk.attention_cached(r.standard_normal((512, d)).astype(np.float32))
+    xs = [r.standard_normal((1, d)).astype(np.float32) for _ in range(8)]
+    for x in xs[:4]:
+        blk.attention_cached(x)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        blk.attention_cached(xs[i % 8])
+    us = (time.perf_counter() - t0) / steps * 1e6
+    blk.close()
+    return {"workload": "llama1b_layer_decode_ctx512", "us_per_step": us, "host_pointers": True,
+            "weight_bytes_per_step": 4 * (2 * d * H * hd + 2 * d * KV * hd)}
+
+
 def load_traffic(kernel, workload):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept as a
     committed summary; None until measured."""
@@ -286,6 +308,9 @@ def main():
             w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, T, 7)
             results[name] = w.run_prefill(k_, max(2, W // 4))
             w.close()
+
+    if want("llama1b_layer_decode_ctx512"):
+        results["llama1b_layer_decode_ctx512"] = layer_decode(sa, np, max(20, K // 4))
 
     h = results[head.name]
     line = {

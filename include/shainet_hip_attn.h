@@ -156,6 +156,37 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
  * and QK-norm of Q exactly (llama_block.cr:332-344). */
 int shainet_attn_last_q_rot(shainet_attn_ctx *ctx, float *out, int rows);
 
+/* ---- the attention half of a LlamaBlock, weights included ------------------
+ *
+ * State and behaviour of src/shainet/transformer/llama_block.cr for
+ * attention_cached_cpu (246-299): x [T, d_model] (host) -> Q/K/V projections ->
+ * bias, QK-norm, RoPE, append, causal GQA attention -> output projection ->
+ * [T, d_model] (host), with everything between the two copies on the device.
+ * Weights are row-major [in, out] as the reference keeps them (hf_loader.cr:326-329).
+ * Constructor checks are those of llama_block.cr:80-89 (head_dim 0 = d_model /
+ * num_heads); eps is the QK-norm eps (92).  Setters may be called at any time
+ * before a forward call, as HFLoader does (hf_loader.cr:319-373); a setter after
+ * rows were cached starts a new, empty cache.  Size mismatches of biases and
+ * norm weights are reported by the next forward call with SHAINET_HIP_ERR_ARGUMENT,
+ * where the reference raises ArgumentError (llama_block.cr:587, 618). */
+typedef struct shainet_llama_attn shainet_llama_attn;
+int shainet_llama_attn_create(shainet_llama_attn **out, int d_model, int num_heads, int num_kv_heads, int head_dim,
+                              double eps, double rope_theta);
+int shainet_llama_attn_destroy(shainet_llama_attn *layer);
+int shainet_llama_attn_set_rope(shainet_llama_attn *layer, double rope_theta, const float *rope_freqs);
+int shainet_llama_attn_set_qk_norm(shainet_llama_attn *layer, const float *q_norm, int q_len, const float *k_norm,
+                                   int k_len);
+int shainet_llama_attn_set_bias(shainet_llama_attn *layer, const float *b_q, int q_len, const float *b_k, int k_len,
+                                const float *b_v, int v_len);
+/* w_q [d_model, q_dim], w_k and w_v [d_model, kv_dim], w_o [q_dim, d_model], host; copied to the device (to_gpu!). */
+int shainet_llama_attn_set_weights(shainet_llama_attn *layer, const float *w_q, const float *w_k, const float *w_v,
+                                   const float *w_o);
+/* LlamaBlock#clear_cache! (116-122) and @cache_len. */
+int shainet_llama_attn_clear_cache(shainet_llama_attn *layer);
+int shainet_llama_attn_cache_len(const shainet_llama_attn *layer);
+/* attention_cached_cpu (246-299): x and out are host [new_tokens, d_model]; synchronous. */
+int shainet_llama_attn_forward_cached(shainet_llama_attn *layer, const float *x, int new_tokens, float *out);
+
 /* Kernel timing for benchmarks: while enabled, every shainet_attn_forward call
  * brackets its attention kernel (the split-K decode kernel, the MFMA prefill
  * kernel or the generic kernel; not the prep or combine kernels) with HIP events

@@ -65,7 +65,7 @@ __device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &
   vb = st.work_off[s] - 1 - level;
 }
 
-template <int HD>
+template <int HD, bool SPLIT>
 __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__restrict__ q_rot,
                                                               const float *__restrict__ kc,
                                                               const float *__restrict__ vc,
@@ -87,8 +87,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   // fill the chip, each block's key range is cut into ns chunks that run as separate
   // workgroups and leave partial (max, sum, O) rows for prefill_combine_kernel.
   const int kvh = blockIdx.x % sh.KV;
-  const int chunk = (blockIdx.x / sh.KV) % ns;
-  const int item = blockIdx.x / sh.KV / ns;
+  const int chunk = SPLIT ? (blockIdx.x / sh.KV) % ns : 0;
+  const int item = SPLIT ? blockIdx.x / sh.KV / ns : blockIdx.x / sh.KV;
   int s, vb;
   locate_block(st, item, s, vb);
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   const int wave_hi = wave_active ? S + min(v0 + 31, VR - 1) / g : -1;  // largest
   const int wg_hi = S + min(vb * 128 + 127, VR - 1) / g;
   const int n_tiles = wg_hi / 32 + 1;
-  const int tiles_per_chunk = (n_tiles + ns - 1) / ns;
+  const int tiles_per_chunk = SPLIT ? (n_tiles + ns - 1) / ns : n_tiles;
   const int kt0 = chunk * tiles_per_chunk, kt1 = min(n_tiles, kt0 + tiles_per_chunk);
   const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
   const float *kbase = kc + head_base;
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float mnew = fmaxf(m, mx);
       // a chunk that starts past a row's last visible key leaves that row at -inf
-      const float mref = mnew == -INFINITY ? 0.f : mnew;
+      const float mref = SPLIT && mnew == -INFINITY ? 0.f : mnew;
       const float alpha = fast_exp2((m - mref) * c);
       const float mc = mref * c;
       float psum = 0.f;
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   }
 
   l += __shfl_xor(l, 32);
-  if (ns > 1) {  // unnormalised partial of this key chunk: [128 virtual rows][HD], (max, sum) per row
+  if (SPLIT) {  // unnormalised partial of this key chunk: [128 virtual rows][HD], (max, sum) per row
     const long long pbase = (((long long)item * sh.KV + kvh) * ns + chunk) * 128 + wave * 32 + n;
     float *op = part_o + pbase * HD;
 #pragma unroll
@@ -435,12 +435,21 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
     const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
     if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
   }
-  if (sh.hd == 64)
-    hipLaunchKernelGGL(prefill_mfma_kernel<64>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, part_ml,
-                       st, sh, ns, c);
-  else
-    hipLaunchKernelGGL(prefill_mfma_kernel<128>, grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, part_ml,
-                       st, sh, ns, c);
+#define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                     \
+  hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_>), grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, \
+                     part_ml, st, sh, ns, c)
+  if (sh.hd == 64) {
+    if (ns > 1)
+      SHAINET_LAUNCH_PREFILL(64, true);
+    else
+      SHAINET_LAUNCH_PREFILL(64, false);
+  } else {
+    if (ns > 1)
+      SHAINET_LAUNCH_PREFILL(128, true);
+    else
+      SHAINET_LAUNCH_PREFILL(128, false);
+  }
+#undef SHAINET_LAUNCH_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || ns == 1) return e;
   hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV)), dim3(256), 0, stream, part_o, part_ml,

@@ -82,6 +82,16 @@ hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, 
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);
 
+// y[T,N] = x[T,K] * W[K,N], T <= 16, N % 4 == 0 (the projections of a decode step).
+struct GemvPlan {
+  int rows_per_wave;
+  int splits;             // workgroups along K; partial sums are added in a fixed order
+  size_t partial_floats;  // scratch the launch needs
+};
+GemvPlan plan_gemv(int T, int K, int N);
+hipError_t launch_gemv(const float *x, const float *w, float *y, float *partials, int T, int K, int N,
+                       const GemvPlan &p, hipStream_t stream);
+
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
                                 int num_kv_heads, int head_dim, int capacity, hipStream_t stream);
 

@@ -26,6 +26,13 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 
+}  // namespace
+
+// for the other translation units of the library
+void shainet_hip_set_error(int code, const char *msg) { fail(code, "%s", msg); }
+
+namespace {
+
 int hip_fail(hipError_t e, const char *what) {
   return fail(e == hipErrorOutOfMemory ? SHAINET_HIP_ERR_ALLOC : SHAINET_HIP_ERR_RUNTIME, "%s: %s", what,
               hipGetErrorString(e));

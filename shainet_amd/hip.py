@@ -72,6 +72,16 @@ _SIGNATURES = {
     "shainet_attn_forward": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_int]),
     "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
+    "shainet_llama_attn_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_int, C.c_double,
+                                            C.c_double]),
+    "shainet_llama_attn_destroy": (C.c_int, [C.c_void_p]),
+    "shainet_llama_attn_set_rope": (C.c_int, [C.c_void_p, C.c_double, _f32p]),
+    "shainet_llama_attn_set_qk_norm": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p, C.c_int]),
+    "shainet_llama_attn_set_bias": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p, C.c_int, _f32p, C.c_int]),
+    "shainet_llama_attn_set_weights": (C.c_int, [C.c_void_p, _f32p, _f32p, _f32p, _f32p]),
+    "shainet_llama_attn_clear_cache": (C.c_int, [C.c_void_p]),
+    "shainet_llama_attn_cache_len": (C.c_int, [C.c_void_p]),
+    "shainet_llama_attn_forward_cached": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p]),
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
@@ -325,3 +335,70 @@ class KVCache:
         _check(lib().shainet_kv_cache_read(self._h, seq, kv_head, pos0, n, k.ctypes.data_as(_f32p),
                                            v.ctypes.data_as(_f32p)))
         return k, v
+
+
+class LlamaBlock:
+    """The attention half of the reference's LlamaBlock (llama_block.cr:6-130, 246-299) on the
+    device: same constructor arguments and checks, same settable properties, `clear_cache`,
+    and `attention_cached(x)` = attention_cached_cpu(x), the part of forward_cached between
+    the two RMSNorms.  Matrices are numpy float32, weights in the reference's [in, out] layout."""
+
+    def __init__(self, d_model, num_heads, ff_hidden=None, eps=1e-6, rope_theta=10000.0, num_kv_heads=None,
+                 head_dim=None):
+        num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        self._h = C.c_void_p()
+        _check(lib().shainet_llama_attn_create(C.byref(self._h), d_model, num_heads, num_kv_heads, head_dim or 0,
+                                               eps, rope_theta))
+        self.d_model, self.num_heads, self.num_kv_heads = d_model, num_heads, num_kv_heads
+        self.head_dim = head_dim or d_model // num_heads
+        self.q_dim, self.kv_dim = num_heads * self.head_dim, num_kv_heads * self.head_dim
+        self._rope_theta, self._rope_freqs = rope_theta, None
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().shainet_llama_attn_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def set_weights(self, w_q, w_k, w_v, w_o):
+        import numpy as np
+
+        ws = [np.ascontiguousarray(w, np.float32) for w in (w_q, w_k, w_v, w_o)]
+        shapes = [(self.d_model, self.q_dim), (self.d_model, self.kv_dim), (self.d_model, self.kv_dim),
+                  (self.q_dim, self.d_model)]
+        for w, sh in zip(ws, shapes):
+            if w.shape != sh:
+                raise ArgumentError(f"weight shape {w.shape} != {sh}")
+        _check(lib().shainet_llama_attn_set_weights(self._h, *[w.ctypes.data_as(_f32p) for w in ws]))
+
+    def set_rope(self, rope_theta, rope_freqs=None):
+        _, fp, _ = keep = _f32_arr(rope_freqs)
+        self._rope_theta, self._rope_freqs = rope_theta, keep[0]
+        _check(lib().shainet_llama_attn_set_rope(self._h, rope_theta, fp))
+
+    def set_qk_norm(self, q_norm, k_norm):
+        a, b = _f32_arr(q_norm), _f32_arr(k_norm)
+        _check(lib().shainet_llama_attn_set_qk_norm(self._h, a[1], a[2], b[1], b[2]))
+
+    def set_bias(self, b_q, b_k, b_v):
+        a = [_f32_arr(b) for b in (b_q, b_k, b_v)]
+        _check(lib().shainet_llama_attn_set_bias(self._h, a[0][1], a[0][2], a[1][1], a[1][2], a[2][1], a[2][2]))
+
+    def clear_cache(self):
+        _check(lib().shainet_llama_attn_clear_cache(self._h))
+
+    @property
+    def cache_len(self):
+        return lib().shainet_llama_attn_cache_len(self._h)
+
+    def attention_cached(self, x):
+        import numpy as np
+
+        x = np.ascontiguousarray(x, np.float32)
+        if x.ndim != 2 or x.shape[1] != self.d_model:
+            raise ArgumentError(f"x must be [T, {self.d_model}]")
+        out = np.empty_like(x)
+        _check(lib().shainet_llama_attn_forward_cached(self._h, x.ctypes.data_as(_f32p), x.shape[0],
+                                                       out.ctypes.data_as(_f32p)))
+        return out

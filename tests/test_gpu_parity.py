@@ -407,3 +407,73 @@ def test_device_pointer_mode_matches_host_pointer_mode(hip):
                 outs.append(ctx.forward(cache, *p, [p[0].shape[0]]))
         res.append(np.concatenate(outs))
     assert np.array_equal(res[0], res[1])
+
+
+# ------------------------------------------------------------------ the layer, projections included
+def _layer_pair(hip, d, H, KV, hd, theta, seed, norm=False, bias=False, wscale=0.02):
+    r = np.random.default_rng(seed)
+    blk = hip.LlamaBlock(d, H, eps=1e-6, rope_theta=theta, num_kv_heads=KV, head_dim=hd)
+    ob = orc.Block(d, H, KV, hd, eps=1e-6, rope_theta=theta)
+    hd_ = blk.head_dim
+    ws = [(wscale * r.standard_normal(s)).astype(np.float32)
+          for s in ((d, H * hd_), (d, KV * hd_), (d, KV * hd_), (H * hd_, d))]
+    blk.set_weights(*ws)
+    ob.set_weights(*ws)
+    if norm:
+        qn, kn = ((1 + 0.02 * r.standard_normal(hd_)).astype(np.float32) for _ in range(2))
+        blk.set_qk_norm(qn, kn)
+        ob.set_qk_norm(qn, kn)
+    if bias:
+        bs = [0.3 * r.standard_normal(n * hd_).astype(np.float32) for n in (H, KV, KV)]
+        blk.set_bias(*bs)
+        ob.set_bias(*bs)
+    return blk, ob, r
+
+
+def test_config1_llama1b_attention_layer_with_projections(hip):
+    # BASELINE configs[0]: hidden 2048, 32 Q / 8 KV heads, head_dim 64, theta 5e5, weights ~N(0, 0.02),
+    # x ~N(0,1); cache brought to 512 positions, then one new row at a time.  The oracle's projections
+    # accumulate in fp64 (SimpleMatrix#*), the device's in fp32.
+    blk, ob, r = _layer_pair(hip, 2048, 32, 8, None, 500000.0, seed=1)
+    x = r.standard_normal((512, 2048)).astype(np.float32)
+    rm.assert_close(blk.attention_cached(x), ob.attention_cached(x), ATOL, RTOL, "prefill 512")
+    for i in range(3):
+        x = r.standard_normal((1, 2048)).astype(np.float32)
+        rm.assert_close(blk.attention_cached(x), ob.attention_cached(x), ATOL, RTOL, f"decode {i}")
+    assert blk.cache_len == ob.cache_len == 515
+
+
+@pytest.mark.parametrize("d,H,KV,hd,norm,bias,Ts", [
+    (64, 8, 4, None, False, False, [6, 1, 1, 1]),     # spec/llama_attention_gpu_spec.cr:16-66
+    (32, 4, 2, None, False, False, [290] + [1] * 10),  # :68-104, crosses the initial capacity of 256
+    (128, 8, 2, 64, True, True, [20, 3, 1, 17]),       # explicit head_dim (q_dim != d_model), QK-norm, biases
+    (256, 8, 8, 128, True, False, [33, 1]),
+])
+def test_layer_matches_oracle(hip, d, H, KV, hd, norm, bias, Ts):
+    blk, ob, r = _layer_pair(hip, d, H, KV, hd, 1e6, seed=d + H, norm=norm, bias=bias, wscale=0.1)
+    xs = [r.uniform(-1, 1, (T, d)).astype(np.float32) for T in Ts]
+    first = []
+    for x in xs:
+        got = blk.attention_cached(x)
+        rm.assert_close(got, ob.attention_cached(x), ATOL, RTOL)
+        first.append(got)
+    # rerun after clear: identical results, no stale rows (spec/llama_attention_gpu_spec.cr:90-103)
+    blk.clear_cache()
+    assert blk.cache_len == 0
+    for x, want in zip(xs, first):
+        assert np.array_equal(blk.attention_cached(x), want)
+
+
+def test_layer_argument_errors(hip):
+    with pytest.raises(hip.ArgumentError):
+        hip.LlamaBlock(64, 8, num_kv_heads=3)
+    with pytest.raises(hip.ArgumentError):
+        hip.LlamaBlock(64, 7)
+    blk, ob, r = _layer_pair(hip, 32, 4, 2, None, 1e4, seed=5)
+    blk.set_bias(np.zeros(31), np.zeros(16), np.zeros(16))  # llama_block.cr:587 raises at forward time
+    with pytest.raises(hip.ArgumentError):
+        blk.attention_cached(np.zeros((1, 32), np.float32))
+    blk.set_bias(None, None, None)
+    blk.set_qk_norm(np.ones(7), np.ones(8))                 # llama_block.cr:618
+    with pytest.raises(hip.ArgumentError):
+        blk.attention_cached(np.zeros((1, 32), np.float32))
