@@ -29,6 +29,11 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Scheduling fence that scalar and vector ALU instructions may cross but LDS,
+// MFMA and global-memory instructions may not: keeps operand fetches ahead of the
+// MFMAs that use them, where the source puts them, instead of next to them.
+#define ORDER_LDS_AND_MFMA() __builtin_amdgcn_sched_barrier(0x7)
+
 __device__ __forceinline__ int find_seq(const SeqTable &st, int item, const int *off) {
   int s = 0;
   while (s + 1 < st.n_seqs && item >= off[s + 1]) ++s;
@@ -134,65 +139,134 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
 
+  // Staging registers: a tile travels global memory -> registers during one
+  // iteration and registers -> LDS at the start of the next.
   f32x4 stage_k[LD4], stage_v[LD4];
-  auto load_tile = [&](int kt) {
+  auto load_k = [&](int kt) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
       const int idx = threadIdx.x + 256 * u;
       const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
-      const long long src = (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4;
-      stage_k[u] = *(const f32x4 *)(kbase + src);
-      stage_v[u] = *(const f32x4 *)(vbase + src);
+      stage_k[u] = *(const f32x4 *)(kbase + (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto load_v = [&](int kt) {
+#pragma unroll
+    for (int u = 0; u < LD4; ++u) {
+      const int idx = threadIdx.x + 256 * u;
+      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
+      stage_v[u] = *(const f32x4 *)(vbase + (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4);
+    }
+  };
+  auto store_k = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
       const int idx = threadIdx.x + 256 * u;
       const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
       *(f32x4 *)&Ks[buf][r * KSTR + 4 * c4] = stage_k[u];
+    }
+  };
+  auto store_v = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < LD4; ++u) {
+      const int idx = threadIdx.x + 256 * u;
+      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
       *(f32x4 *)&Vs[buf][r * HD + 4 * c4] = stage_v[u];
     }
   };
 
+  // S^T of one key tile: 32 keys x 32 virtual rows, K from LDS stage `buf`
+  // MFMA operands come from LDS; every fetch is issued PF steps before the MFMAs
+  // that use it, so that the matrix pipe never waits for an LDS round trip.
+  auto scores = [&](int buf) {
+    constexpr int PF = 2;
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    const float *kl = &Ks[buf][n * KSTR + 4 * j];
+    f32x4 kv[NK4];
+#pragma unroll
+    for (int i = 0; i < PF && i < NK4; ++i) kv[i] = *(const f32x4 *)(kl + 8 * i);
+#pragma unroll
+    for (int i = 0; i < NK4; ++i) {
+      if (i + PF < NK4) kv[i + PF] = *(const f32x4 *)(kl + 8 * (i + PF));
+      ORDER_LDS_AND_MFMA();
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[i].x, qr[4 * i + 0], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[i].y, qr[4 * i + 1], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[i].z, qr[4 * i + 2], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[i].w, qr[4 * i + 3], sacc, 0, 0, 0);
+      ORDER_LDS_AND_MFMA();
+    }
+    return sacc;
+  };
+
+  // Software pipeline over the key tiles.  Iteration kt issues the MFMAs of
+  // S^T(kt+1) before the softmax arithmetic of tile kt, so the vector ALU works in
+  // their shadow, then O^T += V^T(kt) P^T(kt).  K runs two tiles ahead of V:
+  //   LDS at the start of iteration kt:  K(kt+1) in Ks[(kt+1)&1], V(kt) in Vs[kt&1];
+  //   registers:                          K(kt+2), V(kt+1), fetched during kt-1.
+  // The iteration first parks those registers in the two LDS stages nobody reads
+  // any more (Ks[kt&1] held K(kt), Vs[(kt+1)&1] held V(kt-1); both were last
+  // read in iteration kt-1), then fetches K(kt+3) and V(kt+2).  One barrier per
+  // iteration, at its end, orders all of this.
+  f32x16 s_cur, s_next;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s_cur[r] = s_next[r] = 0.f;
   if (kt0 < kt1) {
-    load_tile(kt0);
-    store_tile(kt0 & 1);
+    load_k(kt0);
+    load_v(kt0);
+    store_k(kt0 & 1);
+    store_v(kt0 & 1);
+    if (kt0 + 1 < kt1) {
+      load_k(kt0 + 1);
+      load_v(kt0 + 1);
+      store_k((kt0 + 1) & 1);
+    }
   }
   __syncthreads();
+  if (kt0 + 2 < kt1) load_k(kt0 + 2);
+  if (kt0 < kt1 && kt0 * 32 <= wave_hi) s_cur = scores(kt0 & 1);
+  __syncthreads();  // iteration kt0 overwrites Ks[kt0&1]
+
+  // O^T += V^T P^T of one tile; the probabilities are the registers of `p`
+  auto accumulate = [&](const f32x16 &p, int buf) {
+    constexpr int PF = NT == 2 ? 4 : 2;
+    const float *vl = &Vs[buf][4 * j * HD + NT * n];
+    typedef float vrow_t __attribute__((ext_vector_type(NT)));
+    vrow_t vv[16];
+#pragma unroll
+    for (int r = 0; r < PF; ++r) vv[r] = *(const vrow_t *)(vl + (8 * (r >> 2) + (r & 3)) * HD);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if (r + PF < 16) vv[r + PF] = *(const vrow_t *)(vl + (8 * ((r + PF) >> 2) + ((r + PF) & 3)) * HD);
+      ORDER_LDS_AND_MFMA();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[r][t], p[r], o[t], 0, 0, 0);
+      ORDER_LDS_AND_MFMA();
+    }
+  };
+
+  // tiles [0, n_interior) are visible to every row of this wavefront: no masking
+  const int n_interior = wave_active ? (wave_lo + 1) / 32 : 0;
 
   for (int kt = kt0; kt < kt1; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < kt1) load_tile(kt + 1);
-    if (kt * 32 <= wave_hi) {
-      f32x16 sacc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-      const float *kl = &Ks[buf][n * KSTR + 4 * j];
-#pragma unroll
-      for (int i = 0; i < NK4; ++i) {
-        const f32x4 kv = *(const f32x4 *)(kl + 8 * i);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qr[4 * i + 0], sacc, 0, 0, 0);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qr[4 * i + 1], sacc, 0, 0, 0);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qr[4 * i + 2], sacc, 0, 0, 0);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qr[4 * i + 3], sacc, 0, 0, 0);
-      }
-      if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kt * 32 + 8 * (r >> 2) + 4 * j + (r & 3);
-          if (key > lim) sacc[r] = -INFINITY;
-        }
-      }
+    if (kt + 2 < kt1) store_k(buf);
+    if (kt + 1 < kt1) store_v(buf ^ 1);
+    if (kt + 3 < kt1) load_k(kt + 3);
+    if (kt + 2 < kt1) load_v(kt + 2);
+    if (kt + 1 < n_interior && kt + 1 < kt1) {
+      // Hot path, one basic block: the score MFMAs of tile kt+1 and the softmax
+      // arithmetic of tile kt are independent, so the scheduler can interleave them.
+      s_next = scores(buf ^ 1);
+      f32x16 sacc = s_cur;
       float mx = sacc[0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float mnew = fmaxf(m, mx);
-      // a chunk that starts past a row's last visible key leaves that row at -inf
-      const float mref = SPLIT && mnew == -INFINITY ? 0.f : mnew;
-      const float alpha = fast_exp2((m - mref) * c);
-      const float mc = mref * c;
+      const float mnew = fmaxf(m, mx);  // finite: the tile is fully visible
+      const float alpha = fast_exp2((m - mnew) * c);
+      const float mc = mnew * c;
       float psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -200,31 +274,48 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
         psum += sacc[r];
       }
       l = l * alpha + psum;
-      if (__any(mnew != m)) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
+      m = mnew;
+      accumulate(sacc, buf);
+    } else {
+      if (kt + 1 < kt1 && (kt + 1) * 32 <= wave_hi) s_next = scores(buf ^ 1);
+      if (kt * 32 <= wave_hi) {
+        f32x16 sacc = s_cur;
+        if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kt * 32 + 8 * (r >> 2) + 4 * j + (r & 3);
+            if (key > lim) sacc[r] = -INFINITY;
+          }
+        }
+        float mx = sacc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mnew = fmaxf(m, mx);
+        // a chunk that starts past a row's last visible key leaves that row at -inf
+        const float mref = SPLIT && mnew == -INFINITY ? 0.f : mnew;
+        const float alpha = fast_exp2((m - mref) * c);
+        const float mc = mref * c;
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sacc[r] = fast_exp2(sacc[r] * c - mc);
+          psum += sacc[r];
+        }
+        l = l * alpha + psum;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-      }
-      m = mnew;
-      const float *vl = &Vs[buf][4 * j * HD + NT * n];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float *vp = vl + (8 * (r >> 2) + (r & 3)) * HD;
-        if constexpr (NT == 2) {
-          const float2 vv = *(const float2 *)vp;
-          o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, sacc[r], o[0], 0, 0, 0);
-          o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, sacc[r], o[1], 0, 0, 0);
-        } else {
-          const f32x4 vv = *(const f32x4 *)vp;
-          o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, sacc[r], o[0], 0, 0, 0);
-          o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, sacc[r], o[1], 0, 0, 0);
-          o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.z, sacc[r], o[2], 0, 0, 0);
-          o[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.w, sacc[r], o[3], 0, 0, 0);
-        }
+        m = mnew;
+        accumulate(sacc, buf);
       }
     }
-    if (kt + 1 < kt1) store_tile(buf ^ 1);
+    s_cur = s_next;
     __syncthreads();
   }
 

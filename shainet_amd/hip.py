@@ -12,7 +12,8 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
-_SO = os.path.join(_HERE, "lib", "libshainet_hip_kernels.so")
+# SHAINET_HIP_LIB: load another build of the library (kernel experiments)
+_SO = os.environ.get("SHAINET_HIP_LIB") or os.path.join(_HERE, "lib", "libshainet_hip_kernels.so")
 
 MEM_HOST, MEM_DEVICE = 0, 1
 MAX_BATCH = 64
