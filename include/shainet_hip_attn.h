@@ -187,6 +187,77 @@ int shainet_llama_attn_cache_len(const shainet_llama_attn *layer);
 /* attention_cached_cpu (246-299): x and out are host [new_tokens, d_model]; synchronous. */
 int shainet_llama_attn_forward_cached(shainet_llama_attn *layer, const float *x, int new_tokens, float *out);
 
+/* ---- the whole block ---------------------------------------------------------
+ *
+ * LlamaBlock#forward_cached (llama_block.cr:189-196) with a dense SwiGLU
+ * feed-forward: normed = norm1(x); attn = attention_cached(normed); h = x + attn;
+ * out = h + ffn(norm2(h)), with RMSNorm as rms_norm.cr:18-37 (fp64 sum, root and
+ * scaling), SimpleMatrix#+ as simple_matrix.cr:39-48 and SwiGLUFF#forward as
+ * swiglu_ff.cr:76-91 (g / (1 + exp(-g)) * up in fp64), every step on the device.
+ * Argument order follows LlamaBlock.new (llama_block.cr:71-76): eps is both the
+ * RMSNorm eps and the QK-norm eps (92-94); num_kv_heads 0 = num_heads; head_dim 0
+ * = d_model / num_heads.  The mixture-of-experts feed-forward (moe_experts) is not
+ * covered.  Attention weights, biases, QK-norm and RoPE are set on the handle
+ * shainet_llama_block_attn returns. */
+typedef struct shainet_llama_block shainet_llama_block;
+int shainet_llama_block_create(shainet_llama_block **out, int d_model, int num_heads, int ff_hidden, double eps,
+                               double rope_theta, int num_kv_heads, int head_dim);
+int shainet_llama_block_destroy(shainet_llama_block *block);
+shainet_llama_attn *shainet_llama_block_attn(shainet_llama_block *block);
+/* gamma of @norm1 and @norm2, host [d_model] each; null = ones (rms_norm.cr:10). */
+int shainet_llama_block_set_norms(shainet_llama_block *block, const float *norm1_gamma, const float *norm2_gamma);
+/* gate_proj and up_proj [d_model, ff_hidden], down_proj [ff_hidden, d_model], host, [in, out] (swiglu_ff.cr:16-18). */
+int shainet_llama_block_set_ffn(shainet_llama_block *block, const float *gate_proj, const float *up_proj,
+                                const float *down_proj);
+int shainet_llama_block_clear_cache(shainet_llama_block *block);
+int shainet_llama_block_cache_len(const shainet_llama_block *block);
+/* x and out [new_tokens, d_model].  mem = SHAINET_HIP_MEM_HOST: copies in and out, synchronous;
+ * SHAINET_HIP_MEM_DEVICE: device pointers, asynchronous on the block's stream. */
+int shainet_llama_block_forward_cached(shainet_llama_block *block, const float *x, int new_tokens, float *out,
+                                       int mem);
+
+/* ---- the model around the blocks ----------------------------------------------
+ *
+ * Network#run(SimpleMatrix) with use_kv_cache for a LLaMA-family network
+ * (network_run.cr:185-226): token ids -> embedding rows (embedding_layer.cr:129-153)
+ * -> every block's forward_cached -> final RMSNorm (@final_norm, optional) -> last
+ * row x lm_head [d_model, vocab] (1390-1404) -> + bias (221-225).  Activations and
+ * logits stay on the device.  The sampling entry points work on the logits of the
+ * last run: Sampler.greedy (text/sampler.cr:38-53), Sampler#apply_repetition_penalty!
+ * (59-81) and the top-k selection of Sampler#sample (88-116); the temperature
+ * softmax and the draw over the k survivors (118-150) stay with the caller, who
+ * owns the random generator. */
+typedef struct shainet_llama_model shainet_llama_model;
+int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model, int n_layers, int num_heads,
+                               int num_kv_heads, int head_dim, int ff_hidden, double eps, double rope_theta);
+int shainet_llama_model_destroy(shainet_llama_model *model);
+int shainet_llama_model_layers(const shainet_llama_model *model);
+shainet_llama_block *shainet_llama_model_block(shainet_llama_model *model, int layer);
+/* host [vocab, d_model] */
+int shainet_llama_model_set_embedding(shainet_llama_model *model, const float *table);
+/* host [d_model]; null = the network has no final norm */
+int shainet_llama_model_set_final_norm(shainet_llama_model *model, const float *gamma);
+/* host [d_model, vocab] and [vocab] (null = no bias) */
+int shainet_llama_model_set_lm_head(shainet_llama_model *model, const float *weights, const float *bias);
+int shainet_llama_model_clear_cache(shainet_llama_model *model);
+int shainet_llama_model_cache_len(const shainet_llama_model *model);
+/* tokens: host ids [n_tokens], appended to every block's cache.  logits: host [vocab], or null to leave
+ * them on the device (the call is then asynchronous; the sampling calls and _sync wait). */
+int shainet_llama_model_run(shainet_llama_model *model, const int *tokens, int n_tokens, float *logits);
+int shainet_llama_model_sync(shainet_llama_model *model);
+int shainet_llama_model_read_logits(shainet_llama_model *model, float *logits);
+/* replace the device logits row by host values [vocab]: lets the sampling calls run on a row that
+ * was computed or edited elsewhere (the reference's Sampler takes any SimpleMatrix row) */
+int shainet_llama_model_write_logits(shainet_llama_model *model, const float *logits);
+/* argmax over the finite logits, lowest index among equals, 0 when none is finite */
+int shainet_llama_model_greedy(shainet_llama_model *model, int *token);
+/* v > 0 ? v / penalty : v * penalty for each id in order (a repeated id is penalised again); ids outside
+ * [0, vocab) are skipped; penalty 1.0 is a no-op */
+int shainet_llama_model_repetition_penalty(shainet_llama_model *model, const int *recent_ids, int n, double penalty);
+/* the k largest logits (1 <= k <= 256), NaN excluded, descending, equal values by ascending id;
+ * *count = entries written (< k when fewer are eligible) */
+int shainet_llama_model_topk(shainet_llama_model *model, int k, int *ids, float *vals, int *count);
+
 /* Kernel timing for benchmarks: while enabled, every shainet_attn_forward call
  * brackets its attention kernel (the split-K decode kernel, the MFMA prefill
  * kernel or the generic kernel; not the prep or combine kernels) with HIP events

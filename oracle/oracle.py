@@ -76,6 +76,19 @@ def lib():
         L.orc_rope_apply.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_double]
         L.orc_llama3_rope_freqs.argtypes = [C.c_double, C.c_int, C.c_double, C.c_double, C.c_double,
                                             C.c_double, _f32p]
+        _i32p = C.POINTER(C.c_int)
+        L.orc_embed.argtypes = [_f32p, C.c_int, _i32p, C.c_int, C.c_int, _f32p]
+        L.orc_embed.restype = C.c_int
+        L.orc_logits_last.argtypes = [_f32p, C.c_int, C.c_int, _f32p, C.c_double, _f32p, C.c_int, _f32p, _f32p]
+        L.orc_logits_last.restype = None
+        L.orc_greedy.argtypes = [_f32p, C.c_int]
+        L.orc_greedy.restype = C.c_int
+        L.orc_repetition_penalty.argtypes = [_f32p, C.c_int, _i32p, C.c_int, C.c_int, C.c_double]
+        L.orc_repetition_penalty.restype = None
+        L.orc_topk.argtypes = [_f32p, C.c_int, C.c_int, C.c_double, _i32p, C.POINTER(C.c_double)]
+        L.orc_topk.restype = C.c_int
+        L.orc_sample.argtypes = [_f32p, C.c_int, C.c_int, C.c_double, C.c_double]
+        L.orc_sample.restype = C.c_int
         _lib = L
     return _lib
 
@@ -256,3 +269,58 @@ def llama3_rope_freqs(theta, head_dim, factor, low_freq_factor, high_freq_factor
     out = np.empty(head_dim // 2, np.float32)
     lib().orc_llama3_rope_freqs(theta, head_dim, factor, low_freq_factor, high_freq_factor, old_ctx, _p(out))
     return out
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, np.int32).reshape(-1)
+
+
+def embed(table, ids):
+    """EmbeddingLayer#embed_cpu."""
+    table, ids = _f32(table), _i32(ids)
+    out = np.empty((ids.size, table.shape[1]), np.float32)
+    _check(lib().orc_embed(_p(table), table.shape[0], ids.ctypes.data_as(C.POINTER(C.c_int)), ids.size,
+                           table.shape[1], _p(out)))
+    return out
+
+
+def logits_last(h, final_gamma, eps, lm_head, bias=None):
+    """Final norm (None = the network has none), last row x lm_head [d, vocab], + bias."""
+    h, w = _f32(h), _f32(lm_head)
+    g = _f32(final_gamma) if final_gamma is not None else None
+    b = _f32(bias) if bias is not None else None
+    out = np.empty(w.shape[1], np.float32)
+    lib().orc_logits_last(_p(h), h.shape[0], h.shape[1], _p(g) if g is not None else None, eps, _p(w), w.shape[1],
+                          _p(b) if b is not None else None, _p(out))
+    return out
+
+
+def greedy(logits):
+    """Sampler.greedy over one logits row."""
+    x = _f32(logits).reshape(-1)
+    return lib().orc_greedy(_p(x), x.size)
+
+
+def repetition_penalty(logits, recent_ids, penalty, window=None):
+    """Sampler#apply_repetition_penalty!; returns the penalised copy."""
+    x = _f32(logits).reshape(-1).copy()
+    ids = _i32(recent_ids)
+    lib().orc_repetition_penalty(_p(x), x.size, ids.ctypes.data_as(C.POINTER(C.c_int)), ids.size,
+                                 -1 if window is None else window, penalty)
+    return x
+
+
+def topk(logits, k, temperature=1.0):
+    """The selection loop of Sampler#sample: (ids, value / temperature), descending."""
+    x = _f32(logits).reshape(-1)
+    ids = np.empty(k, np.int32)
+    vals = np.empty(k, np.float64)
+    n = lib().orc_topk(_p(x), x.size, k, temperature, ids.ctypes.data_as(C.POINTER(C.c_int)),
+                       vals.ctypes.data_as(C.POINTER(C.c_double)))
+    return ids[:n], vals[:n]
+
+
+def sample(logits, k, temperature, r):
+    """Sampler#sample with the uniform draw `r` handed in."""
+    x = _f32(logits).reshape(-1)
+    return lib().orc_sample(_p(x), x.size, k, temperature, r)

@@ -34,6 +34,13 @@
  *   orc_attention_full       same fixtures and cached == full.
  *   orc_matmul / orc_rmsnorm / orc_swiglu   numpy fp64 closed forms; tiny-llama
  *                            end-to-end hidden states from transformers.
+ *   orc_embed / orc_logits_last   row gather and numpy fp64 closed forms; tiny-llama
+ *                            end-to-end logits from transformers.
+ *   orc_greedy / orc_repetition_penalty / orc_topk / orc_sample
+ *                            every known answer of spec/sampler_spec.cr; brute force
+ *                            (numpy sort) on random rows with ties, NaN and infinities;
+ *                            the empirical distribution of orc_sample against the
+ *                            temperature softmax.
  * The bit patterns of the sequential fp32 sums and of libm's cosf/sinf/exp/pow
  * as Crystal links them can only be pinned by running the reference, which is
  * not possible without a Crystal compiler; they are restated in the same order
@@ -561,4 +568,116 @@ int orc_block_forward(OrcBlock *b, const float *x, int rows, const float *norm1,
   }
   free(normed); free(attn); free(h); free(ff);
   return rc;
+}
+
+/* ------------------------------------------------------------------ */
+/* After the last block: Network#run, src/shainet/basic/network_run.cr:185-226,
+ * and Sampler, src/shainet/text/sampler.cr. */
+
+/* EmbeddingLayer#embed_cpu : src/shainet/text/embedding_layer.cr:129-153. */
+int orc_embed(const float *table, int vocab, const int *ids, int n, int d, float *out) {
+  for (int r = 0; r < n; ++r) {
+    if (ids[r] < 0 || ids[r] >= vocab) return fail(ORC_ERR_ARGUMENT, "token id outside the table (IndexError)");
+    memcpy(out + (size_t)r * d, table + (size_t)ids[r] * d, sizeof(float) * (size_t)d);
+  }
+  return ORC_OK;
+}
+
+/* network_run.cr:205-226 : final norm over all rows (when the network has one),
+ * last row times the [d, vocab] output matrix (safe_output_transform, 1390-1404,
+ * SimpleMatrix#*), then matrix[i, j] += b[0, j] through the fp64 accessors. */
+void orc_logits_last(const float *h, int rows, int d, const float *final_gamma, double eps, const float *w,
+                     int vocab, const float *bias, float *logits) {
+  float *normed = malloc(sizeof(float) * (size_t)rows * d);
+  const float *src = h;
+  if (final_gamma) {
+    orc_rmsnorm(h, final_gamma, normed, rows, d, eps);
+    src = normed;
+  }
+  orc_matmul(src + (size_t)(rows - 1) * d, w, logits, 1, d, vocab);
+  if (bias)
+    for (int j = 0; j < vocab; ++j) logits[j] = (float)((double)logits[j] + (double)bias[j]);
+  free(normed);
+}
+
+/* Sampler.greedy : sampler.cr:38-53. */
+int orc_greedy(const float *logits, int cols) {
+  int best_id = 0;
+  float best = -INFINITY;
+  for (int j = 0; j < cols; ++j) {
+    float v = logits[j];
+    if (isfinite(v) && v > best) {
+      best = v;
+      best_id = j;
+    }
+  }
+  return best_id;
+}
+
+/* Sampler#apply_repetition_penalty! : sampler.cr:59-81.  window < 0 = all ids. */
+void orc_repetition_penalty(float *logits, int cols, const int *ids, int n, int window, double p) {
+  if (p == 1.0) return;
+  int start = window < 0 ? 0 : n - window;
+  if (start < 0) start = 0;
+  for (int i = start; i < n; ++i) {
+    int id = ids[i];
+    if (0 <= id && id < cols) {
+      float v = logits[id];
+      logits[id] = (float)(v > 0 ? (double)v / p : (double)v * p);
+    }
+  }
+}
+
+/* The selection loop of Sampler#sample : sampler.cr:88-116.  A sorted buffer of
+ * at most k (value / temperature, id) pairs, descending; bsearch_index { |x| x < v }
+ * is the first slot holding a smaller value, so equal values keep arrival order.
+ * Returns the number of survivors. */
+int orc_topk(const float *logits, int cols, int k, double t, int *ids, double *vals) {
+  int sz = 0;
+  for (int j = 0; j < cols; ++j) {
+    double v = (double)logits[j] / t;
+    if (isnan(v)) continue;
+    if (sz == k && !(v > vals[k - 1])) continue;
+    int lo = 0, hi = sz; /* first index with vals[i] < v, or sz */
+    while (lo < hi) {
+      int mid = (lo + hi) / 2;
+      if (vals[mid] < v) hi = mid; else lo = mid + 1;
+    }
+    int last = sz < k ? sz : k - 1; /* insert at lo, dropping the tail when full */
+    for (int i = last; i > lo; --i) {
+      vals[i] = vals[i - 1];
+      ids[i] = ids[i - 1];
+    }
+    vals[lo] = v;
+    ids[lo] = j;
+    if (sz < k) ++sz;
+  }
+  return sz;
+}
+
+/* Sampler#sample : sampler.cr:88-150, with the uniform draw r handed in. */
+int orc_sample(const float *logits, int cols, int k, double t, double r) {
+  int *ids = malloc(sizeof(int) * (size_t)k);
+  double *vals = malloc(sizeof(double) * (size_t)k);
+  int szk = orc_topk(logits, cols, k, t, ids, vals);
+  int best_id = 0;
+  if (szk > 0) {
+    double max_val = vals[0], sum = 0.0;
+    for (int i = 0; i < szk; ++i) {
+      vals[i] = exp(vals[i] - max_val);
+      sum += vals[i];
+    }
+    double inv_sum = 1.0 / sum, cumulative = 0.0;
+    best_id = ids[szk - 1];
+    for (int i = 0; i < szk; ++i) {
+      cumulative += vals[i] * inv_sum;
+      if (r <= cumulative) {
+        best_id = ids[i];
+        break;
+      }
+    }
+  }
+  free(ids);
+  free(vals);
+  return best_id;
 }

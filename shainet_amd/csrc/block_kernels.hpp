@@ -1,0 +1,35 @@
+// Launchers of the kernels around attention in a LlamaBlock and after the last
+// block: RMSNorm, residual add, SwiGLU activation, embedding lookup, logits bias,
+// repetition penalty, greedy argmax and top-k selection.  Device pointers only.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace shainet {
+
+// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma   (gamma == nullptr: ones)
+hipError_t launch_rmsnorm(const float *x, const float *gamma, float *out, int rows, int cols, double eps,
+                          hipStream_t stream);
+// out = a + b, n floats
+hipError_t launch_add(const float *a, const float *b, float *out, long long n, hipStream_t stream);
+// hidden[r, j] = silu(gate_up[r, j]) * gate_up[r, ff + j];  gate_up is [rows, 2*ff]
+hipError_t launch_swiglu_act(const float *gate_up, float *hidden, int rows, int ff, hipStream_t stream);
+// out[t, :] = table[tokens[t], :];  the caller has checked 0 <= tokens[t] < vocab
+hipError_t launch_embed(const float *table, const int *tokens, float *out, int n_tokens, int d_model,
+                        hipStream_t stream);
+// logits[j] += bias[j]
+hipError_t launch_add_bias_row(float *logits, const float *bias, int n, hipStream_t stream);
+// Sampler#apply_repetition_penalty! : ids in order, duplicates penalised once per occurrence
+hipError_t launch_repetition_penalty(float *logits, int vocab, const int *ids, int n, double penalty,
+                                     hipStream_t stream);
+
+// Top-k of a logits row, descending by value, ties by ascending index, NaN never
+// selected (Sampler#sample's selection); with finite_only also +-inf are skipped
+// (Sampler.greedy).  scratch: topk_scratch_bytes(vocab, k) bytes.  out_ids /
+// out_vals: k entries; *out_count = entries found (< k when the row has fewer
+// eligible values).
+constexpr int kMaxTopK = 256;
+size_t topk_scratch_bytes(int vocab, int k);
+hipError_t launch_topk(const float *logits, int vocab, int k, bool finite_only, void *scratch, int *out_ids,
+                       float *out_vals, int *out_count, hipStream_t stream);
+
+}  // namespace shainet

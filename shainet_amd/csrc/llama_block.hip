@@ -6,11 +6,9 @@
 // append, causal GQA attention, output projection.  Activations stay in HBM
 // between the steps; only x comes in and the [T, d_model] result goes out.
 //
-// Projections: a hand-written split GEMV for up to 16 rows (decode), rocBLAS
-// SGEMM (the counterpart of the reference's cuBLAS SGEMM, cuda.cr:237-247) for
-// more.  rocBLAS is opened with dlopen on first use so that the library does not
-// depend on it for decode.
-#include <dlfcn.h>
+// The second half of this file adds what LlamaBlock#forward_cached
+// (llama_block.cr:189-196) does around attention: the two RMSNorms, the two
+// residual adds and the dense SwiGLU feed-forward, again all on the device.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -22,77 +20,13 @@
 
 #include "../../include/shainet_hip_attn.h"
 #include "attn_kernels.hpp"
+#include "block_kernels.hpp"
+#include "llama_internal.hpp"
 
 using namespace shainet;
 
-void shainet_hip_set_error(int code, const char *msg);  // capi.hip
-
 namespace {
-
-// ---- rocBLAS through dlopen -------------------------------------------------
-typedef void *rb_handle;
-typedef int (*rb_create_t)(rb_handle *);
-typedef int (*rb_destroy_t)(rb_handle);
-typedef int (*rb_set_stream_t)(rb_handle, hipStream_t);
-typedef int (*rb_sgemm_t)(rb_handle, int, int, int, int, int, const float *, const float *, int, const float *, int,
-                          const float *, float *, int);
-constexpr int kRocblasOpNone = 111;
-
-struct RocBlas {
-  void *lib = nullptr;
-  rb_create_t create = nullptr;
-  rb_destroy_t destroy = nullptr;
-  rb_set_stream_t set_stream = nullptr;
-  rb_sgemm_t sgemm = nullptr;
-  bool tried = false;
-  bool load() {
-    if (tried) return sgemm != nullptr;
-    tried = true;
-    for (const char *name : {"librocblas.so.5", "librocblas.so"}) {
-      lib = dlopen(name, RTLD_LAZY | RTLD_LOCAL);
-      if (lib) break;
-    }
-    if (!lib) return false;
-    create = (rb_create_t)dlsym(lib, "rocblas_create_handle");
-    destroy = (rb_destroy_t)dlsym(lib, "rocblas_destroy_handle");
-    set_stream = (rb_set_stream_t)dlsym(lib, "rocblas_set_stream");
-    sgemm = (rb_sgemm_t)dlsym(lib, "rocblas_sgemm");
-    if (!create || !destroy || !set_stream || !sgemm) sgemm = nullptr;
-    return sgemm != nullptr;
-  }
-};
-RocBlas g_rocblas;
-
-struct DevF {
-  float *p = nullptr;
-  size_t cap = 0;
-  bool reserve(size_t n) {
-    if (n <= cap) return true;
-    size_t want = cap ? cap : 1024;
-    while (want < n) want *= 2;
-    float *np = nullptr;
-    if (hipMalloc((void **)&np, want * sizeof(float)) != hipSuccess) {
-      (void)hipGetLastError();
-      if (hipMalloc((void **)&np, n * sizeof(float)) != hipSuccess) return false;
-      want = n;
-    }
-    if (p) (void)hipFree(p);
-    p = np;
-    cap = want;
-    return true;
-  }
-  void release() {
-    if (p) (void)hipFree(p);
-    p = nullptr;
-    cap = 0;
-  }
-};
-
-int fail(int code, const std::string &msg) {
-  shainet_hip_set_error(code, msg.c_str());
-  return code;
-}
-
+int fail(int code, const std::string &msg) { return llama_fail(code, msg); }
 }  // namespace
 
 struct shainet_llama_attn {
@@ -106,8 +40,8 @@ struct shainet_llama_attn {
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
   int cache_len = 0;  // @cache_len
-  rb_handle blas = nullptr;
-  DevF x, q, k, v, attn, out, gemv_scratch;
+  Projector proj;
+  DevF x, q, k, v, attn, out;
 };
 
 namespace {
@@ -145,38 +79,35 @@ int ensure_context(shainet_llama_attn *l) {
   return SHAINET_HIP_OK;
 }
 
-// y[T,N] = x[T,K] * W[K,N], all row-major on the device.
-int project(shainet_llama_attn *l, const float *x, const float *w, float *y, int T, int K, int N,
-            hipStream_t stream) {
-  if (T <= 16 && (N & 3) == 0) {
-    const GemvPlan p = plan_gemv(T, K, N);
-    if (!l->gemv_scratch.reserve(p.partial_floats)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-    hipError_t e = launch_gemv(x, w, y, l->gemv_scratch.p, T, K, N, p, stream);
-    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemv launch: ") + hipGetErrorString(e));
-    return SHAINET_HIP_OK;
-  }
-  if (!g_rocblas.load()) return fail(SHAINET_HIP_ERR_RUNTIME, "librocblas.so.5 could not be opened for a projection GEMM");
-  if (!l->blas && g_rocblas.create(&l->blas) != 0) return fail(SHAINET_HIP_ERR_RUNTIME, "rocblas_create_handle failed");
-  if (g_rocblas.set_stream(l->blas, stream) != 0) return fail(SHAINET_HIP_ERR_RUNTIME, "rocblas_set_stream failed");
-  // row-major y = x W  <=>  column-major y^T[N,T] = W^T[N,K] x^T[K,T]
-  const float one = 1.0f, zero = 0.0f;
-  const int st = g_rocblas.sgemm(l->blas, kRocblasOpNone, kRocblasOpNone, N, T, K, &one, w, N, x, K, &zero, y, N);
-  if (st != 0) return fail(SHAINET_HIP_ERR_RUNTIME, "rocblas_sgemm failed with status " + std::to_string(st));
-  return SHAINET_HIP_OK;
-}
-
-int upload_weight(float **dst, const float *src, size_t n) {
-  if (*dst) (void)hipFree(*dst);
-  *dst = nullptr;
-  if (hipMalloc((void **)dst, n * sizeof(float)) != hipSuccess) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-  if (hipMemcpy(*dst, src, n * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
-    return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpy of a weight matrix failed");
-  return SHAINET_HIP_OK;
-}
-
 void set_vec(std::vector<float> &v, bool &has, const float *src, int n) {
   has = src != nullptr;
   v.assign(src ? src : nullptr, src ? src + (n > 0 ? n : 0) : nullptr);
+}
+
+// attention_cached_cpu (llama_block.cr:246-299) with x and out on the device,
+// asynchronous on the layer's stream.
+int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out) {
+  if (!l->w_q) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
+  int rc = ensure_context(l);
+  if (rc) return rc;
+  const int total_len = l->cache_len + T;
+  const int cap = shainet_kv_cache_capacity(l->cache);
+  if (total_len > cap) {  // ensure_gpu_cache! (llama_block.cr:497-520): grow by doubling, contents stay on the device
+    rc = shainet_kv_cache_reserve(l->cache, total_len > 2 * cap ? total_len : 2 * cap);
+    if (rc) return rc;
+  }
+  const size_t qd = (size_t)T * l->q_dim, kd = (size_t)T * l->kv_dim;
+  if (!l->q.reserve(qd) || !l->k.reserve(kd) || !l->v.reserve(kd) || !l->attn.reserve(qd))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
+  if ((rc = l->proj.project(x, l->w_q, l->q.p, T, l->d_model, l->q_dim, stream))) return rc;   // llama_block.cr:253
+  if ((rc = l->proj.project(x, l->w_k, l->k.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 254
+  if ((rc = l->proj.project(x, l->w_v, l->v.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 255
+  rc = shainet_attn_forward(l->ctx, l->cache, nullptr, &T, 1, l->q.p, l->k.p, l->v.p, l->attn.p,
+                            SHAINET_HIP_MEM_DEVICE);  // 256-296
+  if (rc) return rc;
+  l->cache_len = total_len;
+  return l->proj.project(l->attn.p, l->w_o, out, T, l->q_dim, l->d_model, stream);  // 298
 }
 
 }  // namespace
@@ -213,10 +144,10 @@ int shainet_llama_attn_create(shainet_llama_attn **out, int d_model, int num_hea
 int shainet_llama_attn_destroy(shainet_llama_attn *l) {
   if (!l) return SHAINET_HIP_OK;
   drop_context(l);
-  if (l->blas && g_rocblas.destroy) g_rocblas.destroy(l->blas);
+  l->proj.release();
   for (float *p : {l->w_q, l->w_k, l->w_v, l->w_o})
     if (p) (void)hipFree(p);
-  for (DevF *b : {&l->x, &l->q, &l->k, &l->v, &l->attn, &l->out, &l->gemv_scratch}) b->release();
+  for (DevF *b : {&l->x, &l->q, &l->k, &l->v, &l->attn, &l->out}) b->release();
   delete l;
   return SHAINET_HIP_OK;
 }
@@ -252,10 +183,10 @@ int shainet_llama_attn_set_weights(shainet_llama_attn *l, const float *w_q, cons
                                    const float *w_o) {
   if (!l || !w_q || !w_k || !w_v || !w_o) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
-  int rc = upload_weight(&l->w_q, w_q, (size_t)l->d_model * l->q_dim);
-  if (!rc) rc = upload_weight(&l->w_k, w_k, (size_t)l->d_model * l->kv_dim);
-  if (!rc) rc = upload_weight(&l->w_v, w_v, (size_t)l->d_model * l->kv_dim);
-  if (!rc) rc = upload_weight(&l->w_o, w_o, (size_t)l->q_dim * l->d_model);
+  int rc = upload_floats(&l->w_q, w_q, (size_t)l->d_model * l->q_dim);
+  if (!rc) rc = upload_floats(&l->w_k, w_k, (size_t)l->d_model * l->kv_dim);
+  if (!rc) rc = upload_floats(&l->w_v, w_v, (size_t)l->d_model * l->kv_dim);
+  if (!rc) rc = upload_floats(&l->w_o, w_o, (size_t)l->q_dim * l->d_model);
   return rc;
 }
 
@@ -272,29 +203,156 @@ int shainet_llama_attn_forward_cached(shainet_llama_attn *l, const float *x, int
   if (!l->w_q) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);  // raises what add_bias! / apply_head_rmsnorm! raise (llama_block.cr:587, 618)
   if (rc) return rc;
-  const int T = new_tokens;
-  const int total_len = l->cache_len + T;
-  const int cap = shainet_kv_cache_capacity(l->cache);
-  if (total_len > cap) {  // ensure_gpu_cache! (llama_block.cr:497-520): grow by doubling, contents stay on the device
-    rc = shainet_kv_cache_reserve(l->cache, total_len > 2 * cap ? total_len : 2 * cap);
-    if (rc) return rc;
-  }
-  const size_t xd = (size_t)T * l->d_model, qd = (size_t)T * l->q_dim, kd = (size_t)T * l->kv_dim;
-  if (!l->x.reserve(xd) || !l->q.reserve(qd) || !l->k.reserve(kd) || !l->v.reserve(kd) || !l->attn.reserve(qd) ||
-      !l->out.reserve(xd))
-    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  const size_t xd = (size_t)new_tokens * l->d_model;
+  if (!l->x.reserve(xd) || !l->out.reserve(xd)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
   if (hipMemcpyAsync(l->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
-  if ((rc = project(l, l->x.p, l->w_q, l->q.p, T, l->d_model, l->q_dim, stream))) return rc;  // llama_block.cr:253
-  if ((rc = project(l, l->x.p, l->w_k, l->k.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 254
-  if ((rc = project(l, l->x.p, l->w_v, l->v.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 255
-  rc = shainet_attn_forward(l->ctx, l->cache, nullptr, &T, 1, l->q.p, l->k.p, l->v.p, l->attn.p,
-                            SHAINET_HIP_MEM_DEVICE);  // 256-296
-  if (rc) return rc;
-  l->cache_len = total_len;
-  if ((rc = project(l, l->attn.p, l->w_o, l->out.p, T, l->q_dim, l->d_model, stream))) return rc;  // 298
+  if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p))) return rc;
   if (hipMemcpyAsync(out, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+      hipStreamSynchronize(stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
+  return SHAINET_HIP_OK;
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// The whole block: LlamaBlock#forward_cached (llama_block.cr:189-196) with a dense
+// SwiGLU feed-forward (swiglu_ff.cr:76-91).
+struct shainet_llama_block {
+  shainet_llama_attn *attn = nullptr;
+  int d_model = 0, ff_hidden = 0;
+  double eps = 1e-6;                                // RMSNorm eps of @norm1 / @norm2 (llama_block.cr:93-94)
+  float *norm1 = nullptr, *norm2 = nullptr;         // device gamma [d_model]; null = ones (rms_norm.cr:10)
+  float *gate_up = nullptr, *down = nullptr;        // device [d_model, 2*ff] (gate | up) and [ff, d_model]
+  DevF x, normed, attn_out, h, gu, hidden, ff, out;
+};
+
+namespace {
+
+// x and out on the device; asynchronous on the block's stream.
+int block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
+  if (!b->gate_up || !b->down) return fail(SHAINET_HIP_ERR_ARGUMENT, "feed-forward weights not set");
+  shainet_llama_attn *l = b->attn;
+  int rc = ensure_context(l);
+  if (rc) return rc;
+  hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
+  const int d = b->d_model, ff = b->ff_hidden;
+  const size_t xd = (size_t)T * d;
+  if (!b->normed.reserve(xd) || !b->attn_out.reserve(xd) || !b->h.reserve(xd) || !b->gu.reserve((size_t)T * 2 * ff) ||
+      !b->hidden.reserve((size_t)T * ff) || !b->ff.reserve(xd))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  hipError_t e = launch_rmsnorm(x, b->norm1, b->normed.p, T, d, b->eps, stream);  // normed = @norm1.forward(x)
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("rmsnorm launch: ") + hipGetErrorString(e));
+  if ((rc = attn_forward_device(l, b->normed.p, T, b->attn_out.p))) return rc;    // attn = attention_cached_cpu(normed)
+  e = launch_add(x, b->attn_out.p, b->h.p, (long long)xd, stream);                // h = x + attn
+  if (e == hipSuccess) e = launch_rmsnorm(b->h.p, b->norm2, b->normed.p, T, d, b->eps, stream);  // normed2
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("block launch: ") + hipGetErrorString(e));
+  // ff_out = @ffn.forward(normed2): gate and up in one product against [d, 2*ff]
+  if ((rc = l->proj.project(b->normed.p, b->gate_up, b->gu.p, T, d, 2 * ff, stream))) return rc;
+  e = launch_swiglu_act(b->gu.p, b->hidden.p, T, ff, stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("swiglu launch: ") + hipGetErrorString(e));
+  if ((rc = l->proj.project(b->hidden.p, b->down, b->ff.p, T, ff, d, stream))) return rc;
+  e = launch_add(b->h.p, b->ff.p, out, (long long)xd, stream);                     // h + ff_out
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("add launch: ") + hipGetErrorString(e));
+  return SHAINET_HIP_OK;
+}
+
+}  // namespace
+
+// used by the model (llama_model.hip)
+int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
+  return block_forward_device(b, x, T, out);
+}
+int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream) {
+  int rc = ensure_context(b->attn);
+  if (rc) return rc;
+  return shainet_attn_set_stream(b->attn->ctx, (void *)stream);
+}
+
+extern "C" {
+
+int shainet_llama_block_create(shainet_llama_block **out, int d_model, int num_heads, int ff_hidden, double eps,
+                               double rope_theta, int num_kv_heads, int head_dim) {
+  if (!out) return fail(SHAINET_HIP_ERR_ARGUMENT, "out is null");
+  *out = nullptr;
+  if (ff_hidden < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "ff_hidden must be positive");
+  if (num_kv_heads == 0) num_kv_heads = num_heads;  // @num_kv_heads = @num_heads (llama_block.cr:73)
+  shainet_llama_attn *a = nullptr;
+  int rc = shainet_llama_attn_create(&a, d_model, num_heads, num_kv_heads, head_dim, eps, rope_theta);
+  if (rc) return rc;
+  shainet_llama_block *b = new (std::nothrow) shainet_llama_block();
+  if (!b) {
+    shainet_llama_attn_destroy(a);
+    return fail(SHAINET_HIP_ERR_ALLOC, "out of host memory");
+  }
+  b->attn = a;
+  b->d_model = d_model;
+  b->ff_hidden = ff_hidden;
+  b->eps = eps;
+  *out = b;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_block_destroy(shainet_llama_block *b) {
+  if (!b) return SHAINET_HIP_OK;
+  shainet_llama_attn_destroy(b->attn);
+  for (float *p : {b->norm1, b->norm2, b->gate_up, b->down})
+    if (p) (void)hipFree(p);
+  for (DevF *f : {&b->x, &b->normed, &b->attn_out, &b->h, &b->gu, &b->hidden, &b->ff, &b->out}) f->release();
+  delete b;
+  return SHAINET_HIP_OK;
+}
+
+shainet_llama_attn *shainet_llama_block_attn(shainet_llama_block *b) { return b ? b->attn : nullptr; }
+
+int shainet_llama_block_set_norms(shainet_llama_block *b, const float *norm1, const float *norm2) {
+  if (!b) return fail(SHAINET_HIP_ERR_ARGUMENT, "block is null");
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  int rc = SHAINET_HIP_OK;
+  float **dst[2] = {&b->norm1, &b->norm2};
+  const float *src[2] = {norm1, norm2};
+  for (int i = 0; i < 2 && !rc; ++i) {
+    if (src[i]) {
+      rc = upload_floats(dst[i], src[i], (size_t)b->d_model);
+    } else if (*dst[i]) {
+      (void)hipFree(*dst[i]);
+      *dst[i] = nullptr;
+    }
+  }
+  return rc;
+}
+
+int shainet_llama_block_set_ffn(shainet_llama_block *b, const float *gate, const float *up, const float *down) {
+  if (!b || !gate || !up || !down) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  int rc = upload_side_by_side(&b->gate_up, gate, b->ff_hidden, up, b->ff_hidden, b->d_model);
+  if (!rc) rc = upload_floats(&b->down, down, (size_t)b->ff_hidden * b->d_model);
+  return rc;
+}
+
+int shainet_llama_block_clear_cache(shainet_llama_block *b) {
+  if (!b) return fail(SHAINET_HIP_ERR_ARGUMENT, "block is null");
+  return shainet_llama_attn_clear_cache(b->attn);
+}
+
+int shainet_llama_block_cache_len(const shainet_llama_block *b) { return b ? b->attn->cache_len : -1; }
+
+int shainet_llama_block_forward_cached(shainet_llama_block *b, const float *x, int new_tokens, float *out, int mem) {
+  if (!b || !x || !out || new_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
+  if (mem != SHAINET_HIP_MEM_HOST && mem != SHAINET_HIP_MEM_DEVICE)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "mem must be SHAINET_HIP_MEM_HOST or SHAINET_HIP_MEM_DEVICE");
+  if (mem == SHAINET_HIP_MEM_DEVICE) return block_forward_device(b, x, new_tokens, out);
+  int rc = ensure_context(b->attn);
+  if (rc) return rc;
+  const size_t xd = (size_t)new_tokens * b->d_model;
+  if (!b->x.reserve(xd) || !b->out.reserve(xd)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  hipStream_t stream = (hipStream_t)shainet_attn_stream(b->attn->ctx);
+  if (hipMemcpyAsync(b->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
+  if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p))) return rc;
+  if (hipMemcpyAsync(out, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
   return SHAINET_HIP_OK;

@@ -1,0 +1,284 @@
+// Host mirror of the decoder-only model around the blocks, as Network#run walks it
+// with use_kv_cache (src/shainet/basic/network_run.cr:185-226): embedding lookup
+// (text/embedding_layer.cr:129-153) -> LlamaBlock#forward_cached per layer ->
+// final RMSNorm over all rows -> last row times the lm_head matrix
+// [d_model, vocab] (1390-1404) -> bias.  The activations never leave the device;
+// the logits stay there too, so that greedy argmax, the repetition penalty and the
+// top-k selection of text/sampler.cr run on them without a copy of the vocab row.
+#include <hip/hip_runtime.h>
+
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/shainet_hip_attn.h"
+#include "block_kernels.hpp"
+#include "llama_internal.hpp"
+
+using namespace shainet;
+
+// llama_block.hip
+int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out);
+int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream);
+
+struct shainet_llama_model {
+  int vocab = 0, d_model = 0;
+  double eps = 1e-6;
+  std::vector<shainet_llama_block *> blocks;
+  float *embedding = nullptr;   // device [vocab, d_model]
+  float *final_norm = nullptr;  // device [d_model]; has_final_norm says whether the step exists (@final_norm)
+  bool has_final_norm = false;
+  float *lm_head = nullptr;     // device [d_model, vocab]
+  float *lm_bias = nullptr;     // device [vocab] or null
+  hipStream_t stream = nullptr;
+  Projector proj;
+  DevF act[2], normed, logits;
+  int *d_tokens = nullptr;
+  size_t d_tokens_cap = 0;
+  bool have_logits = false;
+  // sampler scratch
+  void *topk_scratch = nullptr;
+  size_t topk_scratch_cap = 0;
+  int *d_ids = nullptr;    // kMaxTopK ids, then the count
+  float *d_vals = nullptr;
+};
+
+namespace {
+
+int fail(int code, const std::string &msg) { return llama_fail(code, msg); }
+
+int reserve_ints(int **p, size_t *cap, size_t n) {
+  if (n <= *cap) return SHAINET_HIP_OK;
+  size_t want = *cap ? *cap : 256;
+  while (want < n) want *= 2;
+  int *np = nullptr;
+  if (hipMalloc((void **)&np, want * sizeof(int)) != hipSuccess) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (*p) (void)hipFree(*p);
+  *p = np;
+  *cap = want;
+  return SHAINET_HIP_OK;
+}
+
+int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *vals, int *count) {
+  if (!m->have_logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "no logits: call shainet_llama_model_run first");
+  if (k < 1 || k > kMaxTopK) return fail(SHAINET_HIP_ERR_ARGUMENT, "k must be in [1, 256]");
+  const size_t need = topk_scratch_bytes(m->vocab, k);
+  if (need > m->topk_scratch_cap) {
+    if (m->topk_scratch) (void)hipFree(m->topk_scratch);
+    m->topk_scratch = nullptr;
+    m->topk_scratch_cap = 0;
+    if (hipMalloc(&m->topk_scratch, need) != hipSuccess) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+    m->topk_scratch_cap = need;
+  }
+  if (!m->d_ids) {
+    if (hipMalloc((void **)&m->d_ids, (kMaxTopK + 1) * sizeof(int)) != hipSuccess ||
+        hipMalloc((void **)&m->d_vals, kMaxTopK * sizeof(float)) != hipSuccess)
+      return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  }
+  hipError_t e = launch_topk(m->logits.p, m->vocab, k, finite_only, m->topk_scratch, m->d_ids, m->d_vals,
+                             m->d_ids + kMaxTopK, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("top-k launch: ") + hipGetErrorString(e));
+  int host_ids[kMaxTopK + 1];
+  if (hipMemcpyAsync(host_ids, m->d_ids, (kMaxTopK + 1) * sizeof(int), hipMemcpyDeviceToHost, m->stream) !=
+          hipSuccess ||
+      (vals && hipMemcpyAsync(vals, m->d_vals, k * sizeof(float), hipMemcpyDeviceToHost, m->stream) != hipSuccess) ||
+      hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the selection back failed");
+  *count = host_ids[kMaxTopK];
+  for (int i = 0; i < k; ++i) ids[i] = host_ids[i];
+  return SHAINET_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model, int n_layers, int num_heads,
+                               int num_kv_heads, int head_dim, int ff_hidden, double eps, double rope_theta) {
+  if (!out) return fail(SHAINET_HIP_ERR_ARGUMENT, "out is null");
+  *out = nullptr;
+  if (vocab < 1 || d_model < 1 || n_layers < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "vocab, d_model and n_layers must be positive");
+  shainet_llama_model *m = new (std::nothrow) shainet_llama_model();
+  if (!m) return fail(SHAINET_HIP_ERR_ALLOC, "out of host memory");
+  m->vocab = vocab;
+  m->d_model = d_model;
+  m->eps = eps;
+  for (int i = 0; i < n_layers; ++i) {
+    shainet_llama_block *b = nullptr;
+    int rc = shainet_llama_block_create(&b, d_model, num_heads, ff_hidden, eps, rope_theta, num_kv_heads, head_dim);
+    if (rc) {
+      shainet_llama_model_destroy(m);
+      return rc;
+    }
+    m->blocks.push_back(b);
+  }
+  *out = m;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_destroy(shainet_llama_model *m) {
+  if (!m) return SHAINET_HIP_OK;
+  for (shainet_llama_block *b : m->blocks) shainet_llama_block_destroy(b);
+  for (float *p : {m->embedding, m->final_norm, m->lm_head, m->lm_bias, m->d_vals})
+    if (p) (void)hipFree(p);
+  if (m->d_tokens) (void)hipFree(m->d_tokens);
+  if (m->d_ids) (void)hipFree(m->d_ids);
+  if (m->topk_scratch) (void)hipFree(m->topk_scratch);
+  m->proj.release();
+  for (DevF *f : {&m->act[0], &m->act[1], &m->normed, &m->logits}) f->release();
+  if (m->stream) (void)hipStreamDestroy(m->stream);
+  delete m;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_layers(const shainet_llama_model *m) { return m ? (int)m->blocks.size() : -1; }
+
+shainet_llama_block *shainet_llama_model_block(shainet_llama_model *m, int i) {
+  if (!m || i < 0 || i >= (int)m->blocks.size()) return nullptr;
+  return m->blocks[i];
+}
+
+int shainet_llama_model_set_embedding(shainet_llama_model *m, const float *table) {
+  if (!m || !table) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  return upload_floats(&m->embedding, table, (size_t)m->vocab * m->d_model);
+}
+
+int shainet_llama_model_set_final_norm(shainet_llama_model *m, const float *gamma) {
+  if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
+  m->has_final_norm = gamma != nullptr;
+  if (!gamma) return SHAINET_HIP_OK;
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  return upload_floats(&m->final_norm, gamma, (size_t)m->d_model);
+}
+
+int shainet_llama_model_set_lm_head(shainet_llama_model *m, const float *w, const float *bias) {
+  if (!m || !w) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  int rc = upload_floats(&m->lm_head, w, (size_t)m->d_model * m->vocab);
+  if (rc) return rc;
+  if (bias) return upload_floats(&m->lm_bias, bias, (size_t)m->vocab);
+  if (m->lm_bias) (void)hipFree(m->lm_bias);
+  m->lm_bias = nullptr;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_clear_cache(shainet_llama_model *m) {
+  if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
+  for (shainet_llama_block *b : m->blocks) {
+    int rc = shainet_llama_block_clear_cache(b);
+    if (rc) return rc;
+  }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_cache_len(const shainet_llama_model *m) {
+  return m && !m->blocks.empty() ? shainet_llama_block_cache_len(m->blocks[0]) : -1;
+}
+
+int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tokens, float *logits) {
+  if (!m || !tokens || n_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
+  if (!m->embedding || !m->lm_head) return fail(SHAINET_HIP_ERR_ARGUMENT, "embedding or lm_head not set");
+  for (int i = 0; i < n_tokens; ++i)  // an id outside the table raises IndexError in the reference
+    if (tokens[i] < 0 || tokens[i] >= m->vocab) return fail(SHAINET_HIP_ERR_ARGUMENT, "token id outside the vocabulary");
+  if (!m->stream && hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamCreate failed");
+  const int T = n_tokens, d = m->d_model;
+  int rc = reserve_ints(&m->d_tokens, &m->d_tokens_cap, (size_t)T);
+  if (rc) return rc;
+  if (!m->act[0].reserve((size_t)T * d) || !m->act[1].reserve((size_t)T * d) || !m->normed.reserve((size_t)T * d) ||
+      !m->logits.reserve((size_t)m->vocab))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  m->have_logits = false;
+  // pageable source: the copy has left the host buffer when the call returns
+  if (hipMemcpyAsync(m->d_tokens, tokens, (size_t)T * sizeof(int), hipMemcpyHostToDevice, m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(tokens) failed");
+  hipError_t e = launch_embed(m->embedding, m->d_tokens, m->act[0].p, T, d, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
+  int cur = 0;
+  for (shainet_llama_block *b : m->blocks) {
+    if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
+    if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
+    cur ^= 1;
+  }
+  // the final norm runs over every row in the reference; only the last one is used afterwards
+  const float *last = m->act[cur].p + (size_t)(T - 1) * d;
+  if (m->has_final_norm) {
+    e = launch_rmsnorm(last, m->final_norm, m->normed.p, 1, d, m->eps, m->stream);
+    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("rmsnorm launch: ") + hipGetErrorString(e));
+    last = m->normed.p;
+  }
+  if ((rc = m->proj.project(last, m->lm_head, m->logits.p, 1, d, m->vocab, m->stream))) return rc;
+  if (m->lm_bias) {
+    e = launch_add_bias_row(m->logits.p, m->lm_bias, m->vocab, m->stream);
+    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("bias launch: ") + hipGetErrorString(e));
+  }
+  m->have_logits = true;
+  if (logits) {
+    if (hipMemcpyAsync(logits, m->logits.p, (size_t)m->vocab * sizeof(float), hipMemcpyDeviceToHost, m->stream) !=
+            hipSuccess ||
+        hipStreamSynchronize(m->stream) != hipSuccess)
+      return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
+  }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_sync(shainet_llama_model *m) {
+  if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
+  if (m->stream && hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamSynchronize failed");
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_greedy(shainet_llama_model *m, int *token) {
+  if (!m || !token) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  int id = 0, count = 0;
+  int rc = run_topk(m, 1, true, &id, nullptr, &count);
+  if (rc) return rc;
+  *token = count > 0 ? id : 0;  // best_id starts at 0 (sampler.cr:41)
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_repetition_penalty(shainet_llama_model *m, const int *recent_ids, int n, double penalty) {
+  if (!m || (n > 0 && !recent_ids)) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!m->have_logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "no logits: call shainet_llama_model_run first");
+  if (penalty == 1.0 || n < 1) return SHAINET_HIP_OK;  // sampler.cr:64
+  int rc = reserve_ints(&m->d_tokens, &m->d_tokens_cap, (size_t)n);
+  if (rc) return rc;
+  if (hipMemcpyAsync(m->d_tokens, recent_ids, (size_t)n * sizeof(int), hipMemcpyHostToDevice, m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(ids) failed");
+  hipError_t e = launch_repetition_penalty(m->logits.p, m->vocab, m->d_tokens, n, penalty, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("penalty launch: ") + hipGetErrorString(e));
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_topk(shainet_llama_model *m, int k, int *ids, float *vals, int *count) {
+  if (!m || !ids || !vals || !count) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  return run_topk(m, k, false, ids, vals, count);
+}
+
+int shainet_llama_model_write_logits(shainet_llama_model *m, const float *logits) {
+  if (!m || !logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  if (!m->stream && hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamCreate failed");
+  if (!m->logits.reserve((size_t)m->vocab)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (hipMemcpyAsync(m->logits.p, logits, (size_t)m->vocab * sizeof(float), hipMemcpyHostToDevice, m->stream) !=
+          hipSuccess ||
+      hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits failed");
+  m->have_logits = true;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_read_logits(shainet_llama_model *m, float *logits) {
+  if (!m || !logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!m->have_logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "no logits: call shainet_llama_model_run first");
+  if (hipMemcpyAsync(logits, m->logits.p, (size_t)m->vocab * sizeof(float), hipMemcpyDeviceToHost, m->stream) !=
+          hipSuccess ||
+      hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
+  return SHAINET_HIP_OK;
+}
+
+}  // extern "C"

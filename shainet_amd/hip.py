@@ -83,6 +83,32 @@ _SIGNATURES = {
     "shainet_llama_attn_clear_cache": (C.c_int, [C.c_void_p]),
     "shainet_llama_attn_cache_len": (C.c_int, [C.c_void_p]),
     "shainet_llama_attn_forward_cached": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p]),
+    "shainet_llama_block_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_double,
+                                             C.c_double, C.c_int, C.c_int]),
+    "shainet_llama_block_destroy": (C.c_int, [C.c_void_p]),
+    "shainet_llama_block_attn": (C.c_void_p, [C.c_void_p]),
+    "shainet_llama_block_set_norms": (C.c_int, [C.c_void_p, _f32p, _f32p]),
+    "shainet_llama_block_set_ffn": (C.c_int, [C.c_void_p, _f32p, _f32p, _f32p]),
+    "shainet_llama_block_clear_cache": (C.c_int, [C.c_void_p]),
+    "shainet_llama_block_cache_len": (C.c_int, [C.c_void_p]),
+    "shainet_llama_block_forward_cached": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]),
+    "shainet_llama_model_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                             C.c_int, C.c_int, C.c_double, C.c_double]),
+    "shainet_llama_model_destroy": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_layers": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_block": (C.c_void_p, [C.c_void_p, C.c_int]),
+    "shainet_llama_model_set_embedding": (C.c_int, [C.c_void_p, _f32p]),
+    "shainet_llama_model_set_final_norm": (C.c_int, [C.c_void_p, _f32p]),
+    "shainet_llama_model_set_lm_head": (C.c_int, [C.c_void_p, _f32p, _f32p]),
+    "shainet_llama_model_clear_cache": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_cache_len": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, _f32p]),
+    "shainet_llama_model_sync": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_read_logits": (C.c_int, [C.c_void_p, _f32p]),
+    "shainet_llama_model_write_logits": (C.c_int, [C.c_void_p, _f32p]),
+    "shainet_llama_model_greedy": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
+    "shainet_llama_model_repetition_penalty": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_double]),
+    "shainet_llama_model_topk": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), _f32p, C.POINTER(C.c_int)]),
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
@@ -339,26 +365,43 @@ class KVCache:
 
 
 class LlamaBlock:
-    """The attention half of the reference's LlamaBlock (llama_block.cr:6-130, 246-299) on the
-    device: same constructor arguments and checks, same settable properties, `clear_cache`,
-    and `attention_cached(x)` = attention_cached_cpu(x), the part of forward_cached between
-    the two RMSNorms.  Matrices are numpy float32, weights in the reference's [in, out] layout."""
+    """The reference's LlamaBlock (llama_block.cr:6-130, 189-196, 246-299) on the device: same
+    constructor arguments and checks, same settable properties, `clear_cache`,
+    `attention_cached(x)` = attention_cached_cpu(x) and, when `ff_hidden` is given,
+    `forward_cached(x)` with the two RMSNorms, the residual adds and the dense SwiGLU
+    feed-forward.  Matrices are numpy float32, weights in the reference's [in, out] layout."""
 
     def __init__(self, d_model, num_heads, ff_hidden=None, eps=1e-6, rope_theta=10000.0, num_kv_heads=None,
-                 head_dim=None):
+                 head_dim=None, _borrowed=None):
         num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
         self._h = C.c_void_p()
-        _check(lib().shainet_llama_attn_create(C.byref(self._h), d_model, num_heads, num_kv_heads, head_dim or 0,
-                                               eps, rope_theta))
-        self.d_model, self.num_heads, self.num_kv_heads = d_model, num_heads, num_kv_heads
+        self._block = None
+        self._owns = _borrowed is None
+        if _borrowed is not None:  # a block owned by a LlamaModel
+            self._block = C.c_void_p(_borrowed)
+            self._h = C.c_void_p(lib().shainet_llama_block_attn(self._block))
+        elif ff_hidden is None:
+            _check(lib().shainet_llama_attn_create(C.byref(self._h), d_model, num_heads, num_kv_heads, head_dim or 0,
+                                                   eps, rope_theta))
+        else:
+            self._block = C.c_void_p()
+            _check(lib().shainet_llama_block_create(C.byref(self._block), d_model, num_heads, ff_hidden, eps,
+                                                    rope_theta, num_kv_heads, head_dim or 0))
+            self._h = C.c_void_p(lib().shainet_llama_block_attn(self._block))
+        self.d_model, self.num_heads, self.num_kv_heads, self.ff_hidden = d_model, num_heads, num_kv_heads, ff_hidden
         self.head_dim = head_dim or d_model // num_heads
         self.q_dim, self.kv_dim = num_heads * self.head_dim, num_kv_heads * self.head_dim
         self._rope_theta, self._rope_freqs = rope_theta, None
 
     def close(self):
-        if getattr(self, "_h", None):
-            lib().shainet_llama_attn_destroy(self._h)
+        if getattr(self, "_h", None) and lib is not None:
+            if self._owns:
+                if self._block is not None:
+                    lib().shainet_llama_block_destroy(self._block)
+                else:
+                    lib().shainet_llama_attn_destroy(self._h)
             self._h = None
+            self._block = None
 
     __del__ = close
 
@@ -386,6 +429,30 @@ class LlamaBlock:
         a = [_f32_arr(b) for b in (b_q, b_k, b_v)]
         _check(lib().shainet_llama_attn_set_bias(self._h, a[0][1], a[0][2], a[1][1], a[1][2], a[2][1], a[2][2]))
 
+    def _need_block(self):
+        if self._block is None:
+            raise ArgumentError("this LlamaBlock was built without ff_hidden: attention only")
+
+    def set_norms(self, norm1_gamma, norm2_gamma):
+        """gamma of @norm1 / @norm2 ([d_model] each; None = ones)."""
+        self._need_block()
+        a, b = _f32_arr(norm1_gamma), _f32_arr(norm2_gamma)
+        for arr in (a, b):
+            if arr[0] is not None and arr[2] != self.d_model:
+                raise ArgumentError(f"norm gamma must have {self.d_model} entries")
+        _check(lib().shainet_llama_block_set_norms(self._block, a[1], b[1]))
+
+    def set_ffn(self, gate_proj, up_proj, down_proj):
+        import numpy as np
+
+        self._need_block()
+        ws = [np.ascontiguousarray(w, np.float32) for w in (gate_proj, up_proj, down_proj)]
+        shapes = [(self.d_model, self.ff_hidden), (self.d_model, self.ff_hidden), (self.ff_hidden, self.d_model)]
+        for w, sh in zip(ws, shapes):
+            if w.shape != sh:
+                raise ArgumentError(f"weight shape {w.shape} != {sh}")
+        _check(lib().shainet_llama_block_set_ffn(self._block, *[w.ctypes.data_as(_f32p) for w in ws]))
+
     def clear_cache(self):
         _check(lib().shainet_llama_attn_clear_cache(self._h))
 
@@ -403,3 +470,175 @@ class LlamaBlock:
         _check(lib().shainet_llama_attn_forward_cached(self._h, x.ctypes.data_as(_f32p), x.shape[0],
                                                        out.ctypes.data_as(_f32p)))
         return out
+
+    def forward_cached(self, x, out=None):
+        """LlamaBlock#forward_cached.  numpy in -> numpy out (copies, synchronous); a CUDA torch
+        tensor in -> torch tensor out (device pointers, asynchronous on the block's stream)."""
+        import numpy as np
+
+        self._need_block()
+        if hasattr(x, "is_cuda") and x.is_cuda:
+            import torch
+
+            if x.dim() != 2 or x.shape[1] != self.d_model or x.dtype != torch.float32 or not x.is_contiguous():
+                raise ArgumentError(f"x must be a contiguous float32 [T, {self.d_model}] tensor")
+            out = torch.empty_like(x) if out is None else out
+            _check(lib().shainet_llama_block_forward_cached(self._block, x.data_ptr(), x.shape[0], out.data_ptr(),
+                                                            MEM_DEVICE))
+            return out
+        x = np.ascontiguousarray(x, np.float32)
+        if x.ndim != 2 or x.shape[1] != self.d_model:
+            raise ArgumentError(f"x must be [T, {self.d_model}]")
+        out = np.empty_like(x)
+        _check(lib().shainet_llama_block_forward_cached(self._block, x.ctypes.data, x.shape[0], out.ctypes.data,
+                                                        MEM_HOST))
+        return out
+
+
+class LlamaModel:
+    """Network#run with use_kv_cache for a LLaMA-family network (network_run.cr:185-226) on the
+    device: embedding -> blocks -> final norm -> lm_head (+ bias), logits kept on the device for
+    `Sampler`."""
+
+    def __init__(self, vocab, d_model, n_layers, num_heads, ff_hidden, eps=1e-6, rope_theta=10000.0,
+                 num_kv_heads=None, head_dim=None):
+        num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
+        self._h = C.c_void_p()
+        _check(lib().shainet_llama_model_create(C.byref(self._h), vocab, d_model, n_layers, num_heads, num_kv_heads,
+                                                head_dim or 0, ff_hidden, eps, rope_theta))
+        self.vocab, self.d_model, self.n_layers = vocab, d_model, n_layers
+        self.blocks = [LlamaBlock(d_model, num_heads, ff_hidden, eps, rope_theta, num_kv_heads, head_dim,
+                                  _borrowed=lib().shainet_llama_model_block(self._h, i)) for i in range(n_layers)]
+
+    def close(self):
+        if getattr(self, "_h", None) and lib is not None:
+            for b in self.blocks:
+                b.close()
+            lib().shainet_llama_model_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def set_embedding(self, table):
+        import numpy as np
+
+        t = np.ascontiguousarray(table, np.float32)
+        if t.shape != (self.vocab, self.d_model):
+            raise ArgumentError(f"embedding shape {t.shape} != {(self.vocab, self.d_model)}")
+        _check(lib().shainet_llama_model_set_embedding(self._h, t.ctypes.data_as(_f32p)))
+
+    def set_final_norm(self, gamma):
+        a = _f32_arr(gamma)
+        if a[0] is not None and a[2] != self.d_model:
+            raise ArgumentError(f"norm gamma must have {self.d_model} entries")
+        _check(lib().shainet_llama_model_set_final_norm(self._h, a[1]))
+
+    def set_lm_head(self, weights, bias=None):
+        import numpy as np
+
+        w = np.ascontiguousarray(weights, np.float32)
+        if w.shape != (self.d_model, self.vocab):
+            raise ArgumentError(f"lm_head shape {w.shape} != {(self.d_model, self.vocab)}")
+        b = _f32_arr(bias)
+        if b[0] is not None and b[2] != self.vocab:
+            raise ArgumentError(f"lm_head bias must have {self.vocab} entries")
+        _check(lib().shainet_llama_model_set_lm_head(self._h, w.ctypes.data_as(_f32p), b[1]))
+
+    def clear_cache(self):
+        _check(lib().shainet_llama_model_clear_cache(self._h))
+
+    @property
+    def cache_len(self):
+        return lib().shainet_llama_model_cache_len(self._h)
+
+    def run(self, tokens, want_logits=True):
+        """Appends `tokens` to the caches; returns the logits row [vocab] of the last token
+        (numpy), or None with want_logits=False (they stay on the device for the Sampler)."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(tokens, np.int32).reshape(-1)
+        logits = np.empty(self.vocab, np.float32) if want_logits else None
+        _check(lib().shainet_llama_model_run(self._h, ids.ctypes.data_as(C.POINTER(C.c_int)), ids.size,
+                                             logits.ctypes.data_as(_f32p) if want_logits else None))
+        return logits
+
+    def sync(self):
+        _check(lib().shainet_llama_model_sync(self._h))
+
+    def logits(self):
+        import numpy as np
+
+        out = np.empty(self.vocab, np.float32)
+        _check(lib().shainet_llama_model_read_logits(self._h, out.ctypes.data_as(_f32p)))
+        return out
+
+    def set_logits(self, row):
+        """Replace the device logits row (e.g. to sample from a row computed elsewhere)."""
+        import numpy as np
+
+        r = np.ascontiguousarray(row, np.float32).reshape(-1)
+        if r.size != self.vocab:
+            raise ArgumentError(f"logits row must have {self.vocab} entries")
+        _check(lib().shainet_llama_model_write_logits(self._h, r.ctypes.data_as(_f32p)))
+
+
+class Sampler:
+    """text/sampler.cr over the device logits of a LlamaModel's last run: greedy, repetition
+    penalty and the top-k selection run on the device; the temperature softmax over the k
+    survivors and the inverse-CDF draw (sampler.cr:118-150) run here in fp64 with `rng`
+    (anything with a `random()` method returning a float in [0, 1))."""
+
+    def __init__(self, temperature=1.0, top_k=40, repetition_penalty=1.0, rng=None):
+        import random
+
+        if top_k < 1:
+            raise ArgumentError("top_k must be >= 1")
+        if not temperature > 0.0:
+            raise ArgumentError("temperature must be > 0")
+        self.temperature, self.top_k, self.repetition_penalty = temperature, top_k, repetition_penalty
+        self.rng = rng if rng is not None else random.Random()
+
+    @staticmethod
+    def greedy(model):
+        tok = C.c_int()
+        _check(lib().shainet_llama_model_greedy(model._h, C.byref(tok)))
+        return tok.value
+
+    def apply_repetition_penalty(self, model, recent_ids, window=None):
+        import numpy as np
+
+        ids = np.ascontiguousarray(recent_ids, np.int32).reshape(-1)
+        if window is not None:
+            ids = np.ascontiguousarray(ids[max(0, ids.size - window):])
+        _check(lib().shainet_llama_model_repetition_penalty(model._h, ids.ctypes.data_as(C.POINTER(C.c_int)),
+                                                            ids.size, self.repetition_penalty))
+
+    def top_candidates(self, model):
+        import numpy as np
+
+        k = self.top_k
+        ids = np.empty(k, np.int32)
+        vals = np.empty(k, np.float32)
+        n = C.c_int()
+        _check(lib().shainet_llama_model_topk(model._h, k, ids.ctypes.data_as(C.POINTER(C.c_int)),
+                                              vals.ctypes.data_as(_f32p), C.byref(n)))
+        return ids[:n.value], vals[:n.value]
+
+    def sample(self, model):
+        import math
+
+        ids, vals = self.top_candidates(model)
+        if len(ids) == 0:
+            return 0  # all-NaN row (sampler.cr:114)
+        v = [float(x) / self.temperature for x in vals]
+        e = [math.exp(x - v[0]) for x in v]  # descending order: element 0 is the max
+        inv = 1.0 / sum(e)
+        r = self.rng.random()
+        cumulative = 0.0
+        best = int(ids[-1])
+        for i, ex in enumerate(e):
+            cumulative += ex * inv
+            if r <= cumulative:
+                best = int(ids[i])
+                break
+        return best

@@ -132,6 +132,36 @@ def tiny_llama_fixture():
     print("wrote tiny_llama_hidden", {k: getattr(v, "shape", None) for k, v in d.items()})
 
 
+def tiny_llama_logits_fixture():
+    """Logits of the reference's tiny-llama data fixture for the token prefixes that
+    spec/llama_loader_spec.cr runs ([1, 42, 100] and one more token), from transformers'
+    LlamaForCausalLM in fp64; the safetensors file and its config are copied next to
+    this script as data (nothing in them is executed)."""
+    import shutil
+
+    from safetensors.torch import load_file
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    dst = os.path.join(HERE, "tiny-llama")
+    os.makedirs(dst, exist_ok=True)
+    for f in ("config.json", "model.safetensors"):
+        shutil.copyfile(os.path.join(TINY, f), os.path.join(dst, f))
+    cfg = LlamaConfig.from_pretrained(TINY)
+    cfg._attn_implementation = "eager"
+    model = LlamaForCausalLM(cfg).eval()
+    res = model.load_state_dict(load_file(os.path.join(TINY, "model.safetensors")), strict=False)
+    assert not res.missing_keys, res
+    model = model.double()
+    d = {}
+    for name, tokens in (("t3", [1, 42, 100]), ("t4", [1, 42, 100, 7])):
+        with torch.no_grad():
+            logits = model(torch.tensor([tokens])).logits[0, -1]
+        d["tokens_" + name] = np.array(tokens, np.int32)
+        d["logits_" + name] = logits.numpy().astype(np.float64)
+    np.savez_compressed(os.path.join(HERE, "tiny_llama_logits.npz"), **d)
+    print("wrote tiny_llama_logits", {k: getattr(v, "shape", None) for k, v in d.items()})
+
+
 def rope_freq_fixture():
     """inv_freq of the published Llama-3.2-1B (hd 64, factor 32) and Llama-3.1-8B (hd 128,
     factor 8) rope_scaling blocks, from transformers' llama3 rope initialiser."""
@@ -172,6 +202,7 @@ def main():
     rope_freq_fixture()
     if os.path.isdir(TINY):
         tiny_llama_fixture()
+        tiny_llama_logits_fixture()
     else:
         print("tiny-llama fixture directory not found; skipped", file=sys.stderr)
 

@@ -1,0 +1,241 @@
+"""Parity of the whole LlamaBlock, of the model around it and of the device sampler with the
+CPU oracle, through the C ABI, on a real MI355X.
+
+Bar (fp32): |gpu - oracle| <= 1e-4 + 1e-3*|oracle| elementwise for activations and logits
+(the oracle's matrix products accumulate in fp64 as SimpleMatrix#* does, the device's in
+fp32); token ids, top-k selections and penalised logits are exact.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import refmath as rm
+import tinyllama
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 1e-4, 1e-3
+NAN, INF = float("nan"), float("inf")
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import shainet_amd as sa
+
+    assert sa.HIP.fully_available(), "no gfx950 device or libshainet_hip_kernels.so missing"
+    return sa
+
+
+def _block_pair(hip, d, H, KV, hd, ff, theta, seed, norm=False, bias=False, wscale=0.05, eps=1e-6):
+    r = np.random.default_rng(seed)
+    blk = hip.LlamaBlock(d, H, ff, eps=eps, rope_theta=theta, num_kv_heads=KV, head_dim=hd)
+    ob = orc.Block(d, H, KV, hd, eps=eps, rope_theta=theta)
+    hd_ = blk.head_dim
+    ws = [(wscale * r.standard_normal(s)).astype(np.float32)
+          for s in ((d, H * hd_), (d, KV * hd_), (d, KV * hd_), (H * hd_, d))]
+    blk.set_weights(*ws)
+    ob.set_weights(*ws)
+    if norm:
+        qn, kn = ((1 + 0.02 * r.standard_normal(hd_)).astype(np.float32) for _ in range(2))
+        blk.set_qk_norm(qn, kn)
+        ob.set_qk_norm(qn, kn)
+    if bias:
+        bs = [0.3 * r.standard_normal(n * hd_).astype(np.float32) for n in (H, KV, KV)]
+        blk.set_bias(*bs)
+        ob.set_bias(*bs)
+    p = {"norm1": (1 + 0.1 * r.standard_normal(d)).astype(np.float32),
+         "norm2": (1 + 0.1 * r.standard_normal(d)).astype(np.float32),
+         "gate": (wscale * r.standard_normal((d, ff))).astype(np.float32),
+         "up": (wscale * r.standard_normal((d, ff))).astype(np.float32),
+         "down": (wscale * r.standard_normal((ff, d))).astype(np.float32)}
+    blk.set_norms(p["norm1"], p["norm2"])
+    blk.set_ffn(p["gate"], p["up"], p["down"])
+    return blk, ob, p, r, eps
+
+
+def _oracle_forward(ob, p, eps, x):
+    return ob.forward(x, p["norm1"], p["norm2"], eps, p["gate"], p["up"], p["down"], True)
+
+
+@pytest.mark.parametrize("d,H,KV,hd,ff,norm,bias,Ts", [
+    (64, 8, 4, None, 96, False, False, [6, 1, 1]),        # odd sizes, generic attention kernel (hd 8)
+    (128, 8, 2, 64, 344, True, True, [20, 3, 1, 17, 1]),  # explicit head_dim, QK-norm, biases, ff % 8 == 0 only
+    (256, 8, 8, 128, 1024, True, False, [33, 1, 1]),
+    (30, 3, 1, None, 50, False, False, [4, 1]),           # widths not multiples of 4: scalar paths, rocBLAS
+])
+def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
+    blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e6, seed=d + ff, norm=norm, bias=bias)
+    for i, T in enumerate(Ts):
+        x = r.standard_normal((T, d)).astype(np.float32)
+        rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, f"call {i} T={T}")
+    assert blk.cache_len == ob.cache_len == sum(Ts)
+    blk.clear_cache()
+    ob.clear_cache()
+    x = r.standard_normal((2, d)).astype(np.float32)
+    rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, "after clear")
+
+
+def test_block_llama1b_shape_prefill_and_decode(hip):
+    # Llama-3.2-1B block: hidden 2048, 32 Q / 8 KV heads, head_dim 64, ff 8192, theta 5e5
+    blk, ob, p, r, eps = _block_pair(hip, 2048, 32, 8, None, 8192, 500000.0, seed=7, wscale=0.02, eps=1e-5)
+    x = r.standard_normal((24, 2048)).astype(np.float32)       # rocBLAS projections (more than 16 rows)
+    rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, "prefill 24")
+    for i in range(2):                                         # split GEMV projections
+        x = r.standard_normal((1, 2048)).astype(np.float32)
+        rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, f"decode {i}")
+
+
+def test_block_device_pointers_match_host_pointers(hip):
+    import torch
+
+    blk, ob, p, r, eps = _block_pair(hip, 128, 8, 2, 64, 256, 1e4, seed=3)
+    x = r.standard_normal((5, 128)).astype(np.float32)
+    want = blk.forward_cached(x)
+    blk.clear_cache()
+    got = blk.forward_cached(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()  # the call is asynchronous on the block's stream
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_block_argument_errors(hip):
+    blk = hip.LlamaBlock(64, 8, 128)
+    with pytest.raises(hip.ArgumentError):
+        blk.forward_cached(np.zeros((1, 64), np.float32))     # nothing set
+    att = hip.LlamaBlock(64, 8)                               # attention only
+    with pytest.raises(hip.ArgumentError):
+        att.forward_cached(np.zeros((1, 64), np.float32))
+    with pytest.raises(hip.ArgumentError):
+        blk.set_ffn(np.zeros((64, 100), np.float32), np.zeros((64, 128), np.float32), np.zeros((128, 64), np.float32))
+
+
+# ---- the model -------------------------------------------------------------------------------
+def _tiny_model(hip):
+    w = tinyllama.load()
+    c = w["cfg"]
+    m = hip.LlamaModel(c["vocab_size"], c["hidden_size"], c["num_hidden_layers"], c["num_attention_heads"],
+                       c["intermediate_size"], eps=c["rms_norm_eps"], rope_theta=c["rope_theta"],
+                       num_kv_heads=c["num_key_value_heads"])
+    m.set_embedding(w["embed"])
+    m.set_final_norm(w["final_norm"])
+    m.set_lm_head(w["lm_head"])
+    for b, lw in zip(m.blocks, w["layers"]):
+        b.set_weights(lw["w_q"], lw["w_k"], lw["w_v"], lw["w_o"])
+        b.set_norms(lw["norm1"], lw["norm2"])
+        b.set_ffn(lw["gate"], lw["up"], lw["down"])
+    return m, w
+
+
+def test_tiny_llama_logits_match_transformers_and_oracle(hip, golden_dir):
+    # the scenario of spec/llama_loader_spec.cr on the reference's own data fixture
+    d = np.load(os.path.join(golden_dir, "tiny_llama_logits.npz"))
+    m, w = _tiny_model(hip)
+    om = tinyllama.OracleModel(w, orc)
+    got3 = m.run(d["tokens_t3"])
+    assert np.abs(got3 - d["logits_t3"]).max() < 1e-5
+    rm.assert_close(got3, om.run(d["tokens_t3"]), ATOL, RTOL, "prefill logits")
+    assert m.cache_len == 3
+    got4 = m.run(d["tokens_t4"][3:])
+    assert np.abs(got4 - d["logits_t4"]).max() < 1e-5
+    rm.assert_close(got4, om.run(d["tokens_t4"][3:]), ATOL, RTOL, "decode logits")
+    assert hip.Sampler.greedy(m) == orc.greedy(got4) == int(np.argmax(d["logits_t4"]))
+    # clear and run the four tokens at once: same last-row logits
+    m.clear_cache()
+    again = m.run(d["tokens_t4"])
+    assert np.abs(again - d["logits_t4"]).max() < 1e-5
+    np.testing.assert_array_equal(m.logits(), again)
+    with pytest.raises(hip.ArgumentError):
+        m.run([32000])
+
+
+def test_tiny_llama_greedy_generation_matches_oracle(hip):
+    m, w = _tiny_model(hip)
+    om = tinyllama.OracleModel(w, orc)
+    toks = [1, 42, 100]
+    m.run(toks, want_logits=False)
+    ol = om.run(toks)
+    for _ in range(12):
+        nxt = hip.Sampler.greedy(m)
+        assert nxt == orc.greedy(ol)
+        m.run([nxt], want_logits=False)
+        ol = om.run([nxt])
+    rm.assert_close(m.logits(), ol, ATOL, RTOL, "logits after 12 generated tokens")
+
+
+# ---- the sampler on the device ---------------------------------------------------------------
+@pytest.fixture(scope="module")
+def sampler_model(hip):
+    # a model used only as the holder of a device logits row of Llama-3's vocabulary size
+    return hip.LlamaModel(128256, 8, 1, 1, 8)
+
+
+def _row(rng, n, special):
+    row = (rng.standard_normal(n) * 3).astype(np.float32)
+    if special:
+        row[rng.integers(0, n, n // 3)] = row[rng.integers(0, n, n // 3)]
+        row[rng.integers(0, n, n // 50 + 1)] = np.nan
+        row[rng.integers(0, n, 3)] = np.inf
+        row[rng.integers(0, n, 3)] = -np.inf
+        row[rng.integers(0, n, 5)] = 0.0
+        row[rng.integers(0, n, 5)] = -0.0
+    return row
+
+
+@pytest.mark.parametrize("seed,special", [(0, False), (1, True), (2, True)])
+def test_device_topk_and_greedy_match_oracle(hip, sampler_model, seed, special):
+    m = sampler_model
+    rng = np.random.default_rng(seed)
+    row = _row(rng, m.vocab, special)
+    m.set_logits(row)
+    assert hip.Sampler.greedy(m) == orc.greedy(row)
+    for k in (1, 5, 40, 256):
+        ids, vals = hip.Sampler(top_k=k).top_candidates(m)
+        want_ids, want_vals = orc.topk(row, k, 1.0)
+        np.testing.assert_array_equal(ids, want_ids)
+        np.testing.assert_array_equal(vals.astype(np.float64), want_vals)
+
+
+def test_device_sampler_known_answers(hip):
+    small = hip.LlamaModel(4, 8, 1, 1, 8)
+    small.set_logits([0.1, 3.2, -1.0, 2.9])
+    assert hip.Sampler.greedy(small) == 1                                      # spec/sampler_spec.cr:11-14
+    small.set_logits([NAN, INF, 0.5, -INF])
+    assert hip.Sampler.greedy(small) == 2                                      # :16-19
+    small.set_logits([NAN, NAN, INF, -INF])
+    assert hip.Sampler.greedy(small) == 0
+    ids, _ = hip.Sampler(top_k=4).top_candidates(small)
+    assert list(ids) == [2, 3]                                                 # NaN out, infinities stay
+    small.set_logits([NAN] * 4)
+    assert hip.Sampler(top_k=3).sample(small) == 0                             # all-NaN row
+    small.set_logits([2.0, -2.0, 0.0, 4.0])
+    hip.Sampler(repetition_penalty=2.0).apply_repetition_penalty(small, [0, 1, 3])   # :65-73
+    np.testing.assert_array_equal(small.logits(), [1.0, -4.0, 0.0, 2.0])
+    hip.Sampler(repetition_penalty=1.0).apply_repetition_penalty(small, [0, 1, 3])   # :75-81
+    np.testing.assert_array_equal(small.logits(), [1.0, -4.0, 0.0, 2.0])
+    small.set_logits([4.0, 4.0, 4.0, 0.0])
+    hip.Sampler(repetition_penalty=2.0).apply_repetition_penalty(small, [0, 1, 2], window=1)  # :83-91
+    np.testing.assert_array_equal(small.logits(), [4.0, 4.0, 2.0, 0.0])
+
+
+def test_device_repetition_penalty_and_sample_match_oracle(hip, sampler_model):
+    m = sampler_model
+    rng = np.random.default_rng(5)
+    row = _row(rng, m.vocab, True)
+    recent = list(rng.integers(0, m.vocab, 60)) + [7, 7, 7, -2, m.vocab + 5]
+    m.set_logits(row)
+    s = hip.Sampler(temperature=0.6, top_k=40, repetition_penalty=1.3)
+    s.apply_repetition_penalty(m, recent, window=50)
+    want = orc.repetition_penalty(row, recent, 1.3, window=50)
+    np.testing.assert_array_equal(m.logits(), want)
+
+    class Fixed:
+        def __init__(self, r):
+            self.r = r
+
+        def random(self):
+            return self.r
+
+    for r in (0.0, 0.03, 0.25, 0.5, 0.77, 0.999999):
+        s.rng = Fixed(r)
+        assert s.sample(m) == orc.sample(want, 40, 0.6, r)
