@@ -200,6 +200,43 @@ def layer_decode(sa, np, steps):
             "weight_bytes_per_step": 4 * (2 * d * H * hd + 2 * d * KV * hd)}
 
 
+def model_decode(sa, np, steps, ctx_len=512):
+    """Greedy decode of a Llama-3.2-1B-shaped model (16 blocks, hidden 2048, 32 Q / 8 KV heads,
+    head_dim 64, ff 8192, vocab 128256, fp32, seeded random weights) with everything on the device:
+    token id in, next token id out.  A token reads every weight once, so the yardstick is weight
+    bytes per token over HBM bandwidth."""
+    r = np.random.default_rng(11)
+    V, d, L, H, KV, hd, ff = 128256, 2048, 16, 32, 8, 64, 8192
+    m = sa.LlamaModel(V, d, L, H, ff, eps=1e-5, rope_theta=5e5, num_kv_heads=KV)
+    table = (0.02 * r.standard_normal((V, d), dtype=np.float32))
+    m.set_embedding(table)
+    m.set_lm_head(table.reshape(d, V))  # same seeded values read as [d, vocab]
+    m.set_final_norm(np.ones(d, np.float32))
+    del table
+    # one block's worth of seeded weights, uploaded into every block (timing does not depend on the values)
+    ws = [(0.02 * r.standard_normal(sh, dtype=np.float32)) for sh in
+          ((d, H * hd), (d, KV * hd), (d, KV * hd), (H * hd, d), (d, ff), (d, ff), (ff, d))]
+    for b in m.blocks:
+        b.set_weights(*ws[:4])
+        b.set_ffn(*ws[4:])
+    del ws
+    weight_bytes = 4 * (L * (2 * d * H * hd + 2 * d * KV * hd + 3 * d * ff) + d * V)
+    m.run(list(r.integers(0, V, ctx_len)), want_logits=False)
+    tok = sa.Sampler.greedy(m)
+    for _ in range(5):
+        m.run([tok], want_logits=False)
+        tok = sa.Sampler.greedy(m)
+    m.run([tok], want_logits=False)
+    m.generate_greedy(16)
+    t0 = time.perf_counter()
+    n = len(m.generate_greedy(steps))
+    dt = (time.perf_counter() - t0) / max(n, 1)
+    m.close()
+    return {"workload": "llama1b_model_greedy_decode_ctx%d" % ctx_len, "us_per_token": dt * 1e6,
+            "tokens_per_s": 1.0 / dt, "weight_bytes_per_token": weight_bytes,
+            "weight_gbps": weight_bytes / dt / 1e9, "frac_of_hbm_peak": weight_bytes / dt / 1e9 / HBM_PEAK_GBPS}
+
+
 def load_traffic(kernel, workload):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept as a
     committed summary; None until measured."""
@@ -311,6 +348,9 @@ def main():
 
     if want("llama1b_layer_decode_ctx512"):
         results["llama1b_layer_decode_ctx512"] = layer_decode(sa, np, max(20, K // 4))
+
+    if want("llama1b_model_greedy_decode_ctx512"):
+        results["llama1b_model_greedy_decode_ctx512"] = model_decode(sa, np, max(20, K // 4))
 
     h = results[head.name]
     line = {

@@ -251,6 +251,15 @@ int shainet_llama_model_read_logits(shainet_llama_model *model, float *logits);
 int shainet_llama_model_write_logits(shainet_llama_model *model, const float *logits);
 /* argmax over the finite logits, lowest index among equals, 0 when none is finite */
 int shainet_llama_model_greedy(shainet_llama_model *model, int *token);
+/* The generation loop of examples/llama_chat.cr:181-197 with greedy selection, kept on the device:
+ * best = Sampler.greedy(logits); stop if best is one of stop_ids; out << best; logits = run([best]);
+ * at most max_tokens times, starting from the logits of the last run.  The chosen id goes from
+ * the argmax kernel to the next step's embedding lookup through device memory, so steps queue up
+ * without a host round trip; the ids are looked at every 16 steps, and when a stop id turns up
+ * the caches are cut back to the rows before it (the logits row is then no longer valid: run
+ * again before sampling).  out: room for max_tokens ids; *n_out = ids written. */
+int shainet_llama_model_generate_greedy(shainet_llama_model *model, int max_tokens, const int *stop_ids, int n_stop,
+                                        int *out, int *n_out);
 /* v > 0 ? v / penalty : v * penalty for each id in order (a repeated id is penalised again); ids outside
  * [0, vocab) are skipped; penalty 1.0 is a no-op */
 int shainet_llama_model_repetition_penalty(shainet_llama_model *model, const int *recent_ids, int n, double penalty);

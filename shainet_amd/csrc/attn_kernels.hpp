@@ -27,6 +27,7 @@ struct Shape {
 
 struct PrepArgs {
   const float *q, *k, *v;           // [tokens, H*hd], [tokens, KV*hd] x2: projection outputs
+  long long q_stride, k_stride, v_stride;  // floats between the rows of two tokens (>= the row width)
   const float *b_q, *b_k, *b_v;     // nullable
   const float *q_norm, *k_norm;     // nullable, [hd]
   double eps;
@@ -82,15 +83,33 @@ hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, 
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);
 
-// y[T,N] = x[T,K] * W[K,N], T <= 16, N % 4 == 0 (the projections of a decode step).
+// y[T,N] = epilogue(norm(x)[T,K] * W[K,N]), T <= 16, N % 4 == 0: the projections of a
+// decode step with what surrounds them fused in.
+enum { kGemvPlain = 0, kGemvResidual = 1, kGemvSwiglu = 2 };
+struct GemvArgs {
+  const float *x;        // [T, K], rows x_stride floats apart
+  long long x_stride;
+  int norm;              // != 0: RMSNorm the rows of x first (gamma may be null = ones)
+  const float *gamma;    // [K]
+  double eps;
+  const float *w;        // [K, N]; kGemvSwiglu: [K, 2N] = gate_proj | up_proj
+  const float *res;      // kGemvResidual: [T, N], y = res + x W
+  float *y;              // [T, N]; kGemvSwiglu: silu(x W_gate) * (x W_up)
+  float *partials;       // GemvPlan::partial_floats floats when the plan has splits > 1
+  int *counters;         // GemvPlan::col_tiles zero-initialised ints, left zero
+  int T, K, N;
+  int epilogue;
+  int rows_per_wave;     // filled in by launch_gemv
+};
 struct GemvPlan {
+  int rows_per_instr;     // 1: 256-column tiles; 4: 64-column tiles, four rows of W per load instruction
   int rows_per_wave;
   int splits;             // workgroups along K; partial sums are added in a fixed order
+  int col_tiles;
   size_t partial_floats;  // scratch the launch needs
 };
-GemvPlan plan_gemv(int T, int K, int N);
-hipError_t launch_gemv(const float *x, const float *w, float *y, float *partials, int T, int K, int N,
-                       const GemvPlan &p, hipStream_t stream);
+GemvPlan plan_gemv(int T, int K, int N, int epilogue);
+hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
 
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
                                 int num_kv_heads, int head_dim, int capacity, hipStream_t stream);

@@ -27,12 +27,13 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 // One workgroup per row.
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
-                                                      float *__restrict__ out, int cols, double eps) {
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x, long long x_stride,
+                                                      const float *__restrict__ gamma, float *__restrict__ out,
+                                                      int cols, double eps) {
   __shared__ double red[4];
-  const float *xr = x + (long long)blockIdx.x * cols;
+  const float *xr = x + (long long)blockIdx.x * x_stride;
   float *orow = out + (long long)blockIdx.x * cols;
-  const bool vec = (cols & 3) == 0;
+  const bool vec = (cols & 3) == 0 && (x_stride & 3) == 0;
   double sq = 0.0;
   if (vec) {
     for (int j = threadIdx.x * 4; j < cols; j += 1024) {
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const float *__restrict
                                                          unsigned long long *__restrict__ cand, int n_cand, int k,
                                                          unsigned long long *__restrict__ winners,
                                                          int *__restrict__ out_ids, float *__restrict__ out_vals,
-                                                         int *__restrict__ out_count) {
+                                                         int *__restrict__ out_count, int fallback_id) {
   // winners[0..k) holds the best so far; each pass selects among them and the next 2048 - 256 candidates
   for (int r = threadIdx.x; r < k; r += 256) winners[r] = 0ull;
   __syncthreads();
@@ -224,13 +225,13 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const float *__restrict
     const unsigned long long key = winners[r];
     if (key != 0ull) {
       out_ids[r] = (int)(~(unsigned)(key & 0xffffffffu));
-      out_vals[r] = key_value(key, logits);
+      if (out_vals) out_vals[r] = key_value(key, logits);
     } else {
-      out_ids[r] = -1;
-      out_vals[r] = 0.f;
+      out_ids[r] = fallback_id;
+      if (out_vals) out_vals[r] = 0.f;
     }
   }
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && out_count) {
     while (count < k && winners[count] != 0ull) ++count;
     *out_count = count;
   }
@@ -238,10 +239,10 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const float *__restrict
 
 }  // namespace
 
-hipError_t launch_rmsnorm(const float *x, const float *gamma, float *out, int rows, int cols, double eps,
-                          hipStream_t stream) {
-  if (rows < 1 || cols < 1) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, stream, x, gamma, out, cols, eps);
+hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
+                          double eps, hipStream_t stream) {
+  if (rows < 1 || cols < 1 || x_stride < cols) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(256), 0, stream, x, x_stride, gamma, out, cols, eps);
   return hipGetLastError();
 }
 
@@ -286,7 +287,7 @@ size_t topk_scratch_bytes(int vocab, int k) {
 }
 
 hipError_t launch_topk(const float *logits, int vocab, int k, bool finite_only, void *scratch, int *out_ids,
-                       float *out_vals, int *out_count, hipStream_t stream) {
+                       float *out_vals, int *out_count, hipStream_t stream, int fallback_id) {
   if (vocab < 1 || k < 1 || k > kMaxTopK || !scratch) return hipErrorInvalidValue;
   const int chunks = (vocab + kTopkChunk - 1) / kTopkChunk;
   unsigned long long *cand = (unsigned long long *)scratch;
@@ -296,7 +297,7 @@ hipError_t launch_topk(const float *logits, int vocab, int k, bool finite_only, 
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(topk_merge_kernel, dim3(1), dim3(256), 0, stream, logits, cand, chunks * k, k, winners, out_ids,
-                     out_vals, out_count);
+                     out_vals, out_count, fallback_id);
   return hipGetLastError();
 }
 

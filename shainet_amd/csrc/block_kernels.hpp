@@ -6,9 +6,10 @@
 
 namespace shainet {
 
-// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma   (gamma == nullptr: ones)
-hipError_t launch_rmsnorm(const float *x, const float *gamma, float *out, int rows, int cols, double eps,
-                          hipStream_t stream);
+// out[r, :] = x[r, :] / sqrt(mean(x[r, :]^2) + eps) * gamma   (gamma == nullptr: ones);
+// the rows of x are x_stride floats apart, those of out are dense
+hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
+                          double eps, hipStream_t stream);
 // out = a + b, n floats
 hipError_t launch_add(const float *a, const float *b, float *out, long long n, hipStream_t stream);
 // hidden[r, j] = silu(gate_up[r, j]) * gate_up[r, ff + j];  gate_up is [rows, 2*ff]
@@ -26,10 +27,11 @@ hipError_t launch_repetition_penalty(float *logits, int vocab, const int *ids, i
 // selected (Sampler#sample's selection); with finite_only also +-inf are skipped
 // (Sampler.greedy).  scratch: topk_scratch_bytes(vocab, k) bytes.  out_ids /
 // out_vals: k entries; *out_count = entries found (< k when the row has fewer
-// eligible values).
+// eligible values); the unused ids are set to fallback_id.  out_vals and out_count
+// may be null.
 constexpr int kMaxTopK = 256;
 size_t topk_scratch_bytes(int vocab, int k);
 hipError_t launch_topk(const float *logits, int vocab, int k, bool finite_only, void *scratch, int *out_ids,
-                       float *out_vals, int *out_count, hipStream_t stream);
+                       float *out_vals, int *out_count, hipStream_t stream, int fallback_id = -1);
 
 }  // namespace shainet

@@ -244,6 +244,10 @@ shainet_attn_ctx *legacy_ctx() {
 
 }  // namespace
 
+int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids,
+                                 const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
+                                 long long q_stride, long long k_stride, long long v_stride, float *out, int mem);
+
 extern "C" {
 
 const char *shainet_hip_last_error(void) { return g_err; }
@@ -524,6 +528,18 @@ int shainet_kv_cache_read(shainet_kv_cache *kc, int seq, int kv_head, int pos0, 
 
 int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, const int *new_tokens,
                          int n_seqs, const float *q, const float *k, const float *v, float *out, int mem) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  return shainet_attn_forward_strided(c, kc, seq_ids, new_tokens, n_seqs, q, k, v, (long long)c->H * c->hd,
+                                      (long long)c->KV * c->hd, (long long)c->KV * c->hd, out, mem);
+}
+
+}  // extern "C"
+
+// The same with the rows of q, k and v at given strides (device pointers): lets a
+// caller hand over the three column blocks of one fused projection output.
+int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids,
+                                 const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
+                                 long long q_stride, long long k_stride, long long v_stride, float *out, int mem) {
   if (!c || !kc || kc->ctx != c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
   if (!new_tokens || !q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (n_seqs < 1 || n_seqs > SHAINET_HIP_MAX_BATCH)
@@ -579,6 +595,9 @@ int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *s
   pa.q = dq;
   pa.k = dk;
   pa.v = dv;
+  pa.q_stride = mem == SHAINET_HIP_MEM_HOST ? (long long)c->H * c->hd : q_stride;
+  pa.k_stride = mem == SHAINET_HIP_MEM_HOST ? (long long)c->KV * c->hd : k_stride;
+  pa.v_stride = mem == SHAINET_HIP_MEM_HOST ? (long long)c->KV * c->hd : v_stride;
   pa.b_q = c->d_bq;
   pa.b_k = c->d_bk;
   pa.b_v = c->d_bv;
@@ -600,6 +619,8 @@ int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *s
   }
   return SHAINET_HIP_OK;
 }
+
+extern "C" {
 
 int shainet_attn_profile(shainet_attn_ctx *c, int enable) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");

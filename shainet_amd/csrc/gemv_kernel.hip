@@ -1,12 +1,23 @@
-// y[T,N] = x[T,K] * W[K,N] for a few rows (T <= 16), fp32: the Q/K/V/O projections
-// of a decode step (llama_block.cr:253-255, 298 with weights in the reference's
-// [in, out] layout).  The product is bound by reading W once from HBM, so the
-// work is cut along K as well as along N to put enough workgroups in flight: a
-// wavefront owns 256 consecutive columns (one float4 per lane, 1 KiB per W row)
-// and a run of rows of W; the four wavefronts of a workgroup take four runs and
-// add up through LDS; a second kernel adds the workgroups' partial sums in a
-// fixed order (no atomics: results do not depend on scheduling).
+// y[T,N] = f(x)[T,K] * W[K,N] for a few rows (T <= 16), fp32: the projections of a
+// decode step (llama_block.cr:253-255, 298; swiglu_ff.cr:76-91; the lm_head product
+// of network_run.cr:1390-1404) with weights in the reference's [in, out] layout.
+//
+// The product is bound by reading W once from HBM, so the work is cut along K as
+// well as along N to put enough workgroups in flight: a wavefront owns 256
+// consecutive columns (one float4 per lane, 1 KiB per W row) and a run of rows of
+// W; the four wavefronts of a workgroup take four runs and add up through LDS.
+// With more than one workgroup along K, each leaves a partial sum and the last one
+// to arrive at a column tile (an atomic counter per tile tells) adds the partials
+// in a fixed order, so results do not depend on scheduling, and applies the
+// epilogue.  Everything a decode step does around a product rides along:
+//   * prologue: RMSNorm of the x rows (rms_norm.cr:18-37, fp64 as there), so the
+//     normalised activations never go to memory;
+//   * epilogue: residual add (simple_matrix.cr:39-48) or the SwiGLU gate
+//     (swiglu_ff.cr:84-89) over a [K, 2*ff] matrix holding gate_proj | up_proj.
 #include "attn_kernels.hpp"
+
+#include <math.h>
+#include <stdlib.h>
 
 namespace shainet {
 
@@ -14,100 +25,288 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-template <int TT>
-__global__ __launch_bounds__(256) void gemv_partial_kernel(const float *__restrict__ x, const float *__restrict__ w,
-                                                           float *__restrict__ part, int T, int K, int N,
-                                                           int rows_per_wave) {
-  __shared__ f32x4 red[4][TT][64];
+// Partial sums cross workgroups that may sit on different XCDs, whose L2 caches
+// are not kept coherent with each other for ordinary accesses: the store is
+// written through to memory (sc1 = device scope), 16 bytes at a time.
+__device__ __forceinline__ void coherent_store4(float *p, f32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+
+__device__ __forceinline__ float swiglu1(float gate, float up) {
+  const double g = (double)gate;
+  return (float)((g / (1.0 + exp(-g))) * (double)up);
+}
+
+__device__ __forceinline__ f32x4 apply_epilogue(int epi, f32x4 a, f32x4 b, const float *res) {
+  if (epi == kGemvSwiglu) return f32x4{swiglu1(a.x, b.x), swiglu1(a.y, b.y), swiglu1(a.z, b.z), swiglu1(a.w, b.w)};
+  if (epi == kGemvResidual) {
+    const f32x4 r = *(const f32x4 *)res;
+    return f32x4{(float)((double)r.x + (double)a.x), (float)((double)r.y + (double)a.y),
+                 (float)((double)r.z + (double)a.z), (float)((double)r.w + (double)a.w)};
+  }
+  return a;
+}
+
+// NACC = 1, or 2 for the SwiGLU epilogue (gate and up accumulators).
+// RPI = rows of W per load instruction: 1 (a wavefront spans 256 columns) or 4
+// (16 lanes per row, 64 columns, four consecutive rows at once).  Narrow tiles give
+// a matrix with few columns enough column tiles that 16 workgroups along K
+// suffice: the arrivals at a tile's counter serialise at roughly 0.1 us each.
+template <int TT, int NACC, int RPI>
+__global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
+  constexpr int LPR = 64 / RPI;  // lanes across a row
+  constexpr int CW = LPR * 4;    // columns per tile
+  extern __shared__ float smem[];  // xs[TT][4 * rows_per_wave]; reused for the cross-wavefront sums
+  __shared__ double rms_s[TT];
+  __shared__ double red_s[4];
+  __shared__ bool last_flag;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col = blockIdx.x * 256 + lane * 4;
-  const int k0 = (blockIdx.y * 4 + wave) * rows_per_wave;
-  const int k1 = min(K, k0 + rows_per_wave);
-  f32x4 acc[TT];
-#pragma unroll
-  for (int t = 0; t < TT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  if (col < N) {  // N is a multiple of 4
-    const float *wp = w + (long long)k0 * N + col;
-    int k = k0;
-    for (; k + 4 <= k1; k += 4) {  // four rows of W in flight
-      f32x4 r[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) r[u] = *(const f32x4 *)(wp + (long long)u * N);
-      wp += 4LL * N;
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int t = 0; t < TT; ++t) {
-          const float xv = t < T ? x[(long long)t * K + k + u] : 0.f;  // uniform over the wavefront
-          acc[t] += xv * r[u];
+  const int cl = lane % LPR, sub = lane / LPR;
+  const int T = a.T, K = a.K, N = a.N;
+  const int rpw = a.rows_per_wave, span = 4 * rpw;  // rpw is a multiple of 8 * RPI
+  const int col = blockIdx.x * CW + cl * 4;
+  const int k_wg = blockIdx.y * span;
+  const int ldw = NACC * N;  // row pitch of W
+  const bool have_col = col < N;  // N is a multiple of 4
+
+  // ---- prologue: the x values of this workgroup's K range, normalised if asked;
+  // zero beyond K and beyond T, so that clamped loads below contribute nothing
+  if (a.norm) {
+    for (int t = 0; t < T; ++t) {
+      const float *xr = a.x + (long long)t * a.x_stride;
+      double sq = 0.0;
+      if (((K | a.x_stride) & 3) == 0) {
+        for (int k = threadIdx.x * 4; k < K; k += 1024) {
+          const f32x4 v = *(const f32x4 *)(xr + k);
+          sq += (double)v.x * (double)v.x + (double)v.y * (double)v.y;
+          sq += (double)v.z * (double)v.z + (double)v.w * (double)v.w;
         }
-    }
-    for (; k < k1; ++k) {
-      const f32x4 r = *(const f32x4 *)wp;
-      wp += N;
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        const float xv = t < T ? x[(long long)t * K + k] : 0.f;
-        acc[t] += xv * r;
+      } else {
+        for (int k = threadIdx.x; k < K; k += 256) sq += (double)xr[k] * (double)xr[k];
       }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+      if (lane == 0) red_s[wave] = sq;
+      __syncthreads();
+      if (threadIdx.x == 0) rms_s[t] = sqrt(((red_s[0] + red_s[1]) + (red_s[2] + red_s[3])) / (double)K + a.eps);
+      __syncthreads();
     }
   }
-#pragma unroll
-  for (int t = 0; t < TT; ++t) red[wave][t][lane] = acc[t];
+  for (int idx = threadIdx.x; idx < TT * span; idx += 256) {
+    const int t = idx / span, kk = idx - t * span, k = k_wg + kk;
+    float v = 0.f;
+    if (t < T && k < K) {
+      v = a.x[(long long)t * a.x_stride + k];
+      if (a.norm) v = (float)(((double)v / rms_s[t]) * (double)(a.gamma ? a.gamma[k] : 1.f));
+    }
+    smem[idx] = v;
+  }
   __syncthreads();
-  if (wave == 0 && col < N) {
+
+  // ---- main loop: eight load instructions (8 * RPI rows of W) in flight per wavefront
+  f32x4 acc[NACC][TT];
+#pragma unroll
+  for (int c = 0; c < NACC; ++c)
+#pragma unroll
+    for (int t = 0; t < TT; ++t) acc[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int kk0 = wave * rpw;  // this wavefront's rows, relative to k_wg
+  if (have_col) {
+    for (int kb = 0; kb < rpw && k_wg + kk0 + kb < K; kb += 8 * RPI) {
+      f32x4 r[NACC][8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int row = min(k_wg + kk0 + kb + u * RPI + sub, K - 1);
+#pragma unroll
+        for (int c = 0; c < NACC; ++c) r[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+          const float xv = smem[t * span + kk0 + kb + u * RPI + sub];  // one address per row: broadcasts
+#pragma unroll
+          for (int c = 0; c < NACC; ++c) acc[c][t] += xv * r[c][u];
+        }
+    }
+  }
+  if constexpr (RPI > 1) {  // add the RPI row groups of the wavefront: every lane ends up with the sum
+#pragma unroll
+    for (int c = 0; c < NACC; ++c)
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+#pragma unroll
+        for (int o = LPR; o < 64; o <<= 1) {
+          acc[c][t].x += __shfl_xor(acc[c][t].x, o);
+          acc[c][t].y += __shfl_xor(acc[c][t].y, o);
+          acc[c][t].z += __shfl_xor(acc[c][t].z, o);
+          acc[c][t].w += __shfl_xor(acc[c][t].w, o);
+        }
+  }
+
+  // ---- the four wavefronts add up through LDS (the x staging area is free now),
+  // one accumulator set at a time to keep the footprint at [3][TT][64] float4
+  f32x4 *red = (f32x4 *)smem;
+  const int splits = gridDim.y;
+#pragma unroll
+  for (int c = 0; c < NACC; ++c) {
+    __syncthreads();
+    if (wave > 0) {
+#pragma unroll
+      for (int t = 0; t < TT; ++t) red[((wave - 1) * TT + t) * 64 + lane] = acc[c][t];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < TT; ++t)
+        acc[c][t] = (acc[c][t] + red[(0 * TT + t) * 64 + lane]) + (red[(1 * TT + t) * 64 + lane] + red[(2 * TT + t) * 64 + lane]);
+    }
+  }
+  if (wave == 0 && sub == 0 && have_col) {
 #pragma unroll
     for (int t = 0; t < TT; ++t)
       if (t < T) {
-        const f32x4 sum = (red[0][t][lane] + red[1][t][lane]) + (red[2][t][lane] + red[3][t][lane]);
-        *(f32x4 *)(part + ((long long)blockIdx.y * T + t) * N + col) = sum;
+        if (splits == 1) {
+          const float *res = a.res ? a.res + (long long)t * N + col : nullptr;
+          *(f32x4 *)(a.y + (long long)t * N + col) = apply_epilogue(a.epilogue, acc[0][t], acc[NACC - 1][t], res);
+        } else {
+#pragma unroll
+          for (int c = 0; c < NACC; ++c)
+            coherent_store4(a.partials + (((long long)blockIdx.y * T + t) * NACC + c) * N + col, acc[c][t]);
+        }
       }
   }
-}
+  if (splits == 1) return;
 
-__global__ __launch_bounds__(256) void gemv_reduce_kernel(const float *__restrict__ part, float *__restrict__ y,
-                                                          int total, int splits) {
-  const int i = blockIdx.x * 256 + threadIdx.x;  // over T*N/4 float4
-  if (i >= total) return;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < splits; ++s) acc += ((const f32x4 *)part)[(long long)s * total + i];
-  ((f32x4 *)y)[i] = acc;
+  // ---- the last workgroup of this column tile adds the partials in a fixed order
+  __syncthreads();  // the partial stores above are acknowledged before the arrival is counted
+  if (threadIdx.x == 0) {
+    const int old = atomicAdd(&a.counters[blockIdx.x], 1);
+    last_flag = old == splits - 1;
+    if (last_flag) atomicExch(&a.counters[blockIdx.x], 0);  // ready for the next launch
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  for (int t = 0; t < T; ++t) {
+    // row group g = wave * RPI + sub adds splits g, g + 4 * RPI, ... (FL loads in flight);
+    // then the groups of a wavefront are added by shuffles and the wavefronts through LDS
+    f32x4 part[NACC];
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) part[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (have_col) {
+      constexpr int FL = NACC == 1 ? 8 : 4;  // loads in flight per lane
+      for (int s0 = wave * RPI + sub; s0 < splits; s0 += 4 * RPI * FL) {
+        f32x4 v[NACC][FL];
+#pragma unroll
+        for (int u = 0; u < FL; ++u) {
+          const int s = min(s0 + 4 * RPI * u, splits - 1);
+#pragma unroll
+          for (int c = 0; c < NACC; ++c)
+            v[c][u] = *(const f32x4 *)(a.partials + (((long long)s * T + t) * NACC + c) * N + col);
+        }
+#pragma unroll
+        for (int u = 0; u < FL; ++u)
+          if (s0 + 4 * RPI * u < splits) {
+#pragma unroll
+            for (int c = 0; c < NACC; ++c) part[c] += v[c][u];
+          }
+      }
+    }
+    if constexpr (RPI > 1) {
+#pragma unroll
+      for (int c = 0; c < NACC; ++c)
+#pragma unroll
+        for (int o = LPR; o < 64; o <<= 1) {
+          part[c].x += __shfl_xor(part[c].x, o);
+          part[c].y += __shfl_xor(part[c].y, o);
+          part[c].z += __shfl_xor(part[c].z, o);
+          part[c].w += __shfl_xor(part[c].w, o);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) red[(wave * NACC + c) * 64 + lane] = part[c];
+    __syncthreads();
+    if (wave == 0 && sub == 0 && have_col) {
+      f32x4 sum[NACC];
+#pragma unroll
+      for (int c = 0; c < NACC; ++c)
+        sum[c] = (red[(0 * NACC + c) * 64 + lane] + red[(1 * NACC + c) * 64 + lane]) +
+                 (red[(2 * NACC + c) * 64 + lane] + red[(3 * NACC + c) * 64 + lane]);
+      const float *res = a.res ? a.res + (long long)t * N + col : nullptr;
+      *(f32x4 *)(a.y + (long long)t * N + col) = apply_epilogue(a.epilogue, sum[0], sum[NACC - 1], res);
+    }
+  }
 }
 
 }  // namespace
 
-GemvPlan plan_gemv(int T, int K, int N) {
+GemvPlan plan_gemv(int T, int K, int N, int epilogue) {
   GemvPlan p;
-  const int col_tiles = (N + 255) / 256;
-  // about 1024 workgroups per product, at least 8 rows of W per wavefront
-  int splits = (1024 + col_tiles - 1) / col_tiles;
+  const int nacc = epilogue == kGemvSwiglu ? 2 : 1;
+  static const int wg_env = getenv("SHAINET_HIP_GEMV_WGS") ? atoi(getenv("SHAINET_HIP_GEMV_WGS")) : 0;
+  // about 1024 workgroups per product (512 when each reads two matrices' worth) but at
+  // most 16 along K; a matrix too narrow for that with 256-column tiles gets 64-column ones
+  const int target = (wg_env > 0 ? wg_env : 1024) / nacc;
+  p.rows_per_instr = ((N + 255) / 256) * 16 < target ? 4 : 1;
+  const int cw = 256 / p.rows_per_instr;
+  const int col_tiles = (N + cw - 1) / cw;
+  int splits = (target + col_tiles - 1) / col_tiles;
+  if (splits > 16) splits = 16;
+  // rows of W per wavefront: a multiple of what eight load instructions cover, at
+  // most 256 or, with more than 4 rows of x, 128 (the x staging area in LDS holds
+  // rows of x * 4 * rows_per_wave floats)
+  const int quantum = 8 * p.rows_per_instr;
+  const int max_rows = T > 4 ? 128 : 256;
   int rows = (K + 4 * splits - 1) / (4 * splits);
-  if (rows < 8) rows = 8;
+  rows = rows / quantum * quantum;
+  if (rows < quantum) rows = quantum;
+  if (rows > max_rows) rows = max_rows;
   splits = (K + 4 * rows - 1) / (4 * rows);
   p.rows_per_wave = rows;
   p.splits = splits;
-  p.partial_floats = (size_t)splits * T * N;
+  p.col_tiles = col_tiles;
+  p.partial_floats = splits > 1 ? (size_t)splits * T * nacc * N : 0;
   return p;
 }
 
-hipError_t launch_gemv(const float *x, const float *w, float *y, float *partials, int T, int K, int N,
-                       const GemvPlan &p, hipStream_t stream) {
-  if (T < 1 || T > 16 || K < 1 || N < 4 || (N & 3) || !partials) return hipErrorInvalidValue;
-  dim3 grid((unsigned)((N + 255) / 256), (unsigned)p.splits);
-#define SHAINET_LAUNCH_GEMV(TT_) \
-  hipLaunchKernelGGL(gemv_partial_kernel<TT_>, grid, dim3(256), 0, stream, x, w, partials, T, K, N, p.rows_per_wave)
-  if (T == 1)
-    SHAINET_LAUNCH_GEMV(1);
-  else if (T <= 4)
-    SHAINET_LAUNCH_GEMV(4);
+hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stream) {
+  GemvArgs a = args;
+  if (a.T < 1 || a.T > 16 || a.K < 1 || a.N < 4 || (a.N & 3) || !a.x || !a.w || !a.y || a.x_stride < a.K)
+    return hipErrorInvalidValue;
+  if (p.rows_per_instr != 1 && p.rows_per_instr != 4) return hipErrorInvalidValue;
+  if (p.rows_per_wave < 8 * p.rows_per_instr || p.rows_per_wave % (8 * p.rows_per_instr)) return hipErrorInvalidValue;
+  if (p.splits > 1 && (!a.partials || !a.counters)) return hipErrorInvalidValue;
+  if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
+  if (a.epilogue != kGemvResidual) a.res = nullptr;
+  a.rows_per_wave = p.rows_per_wave;
+  dim3 grid((unsigned)p.col_tiles, (unsigned)p.splits);
+  const int nacc = a.epilogue == kGemvSwiglu ? 2 : 1;
+  const int tt = a.T == 1 ? 1 : (a.T <= 4 ? 4 : 16);
+  const size_t stage = (size_t)tt * 4 * p.rows_per_wave * sizeof(float);
+  const size_t red = (size_t)(3 * tt > 4 * nacc ? 3 * tt : 4 * nacc) * 64 * sizeof(f32x4);
+  const size_t smem = stage > red ? stage : red;
+#define SHAINET_LAUNCH_GEMV(TT_, NACC_, RPI_) \
+  hipLaunchKernelGGL((gemv_fused_kernel<TT_, NACC_, RPI_>), grid, dim3(256), smem, stream, a)
+#define SHAINET_LAUNCH_GEMV_T(NACC_, RPI_)   \
+  do {                                       \
+    if (tt == 1)                             \
+      SHAINET_LAUNCH_GEMV(1, NACC_, RPI_);   \
+    else if (tt == 4)                        \
+      SHAINET_LAUNCH_GEMV(4, NACC_, RPI_);   \
+    else                                     \
+      SHAINET_LAUNCH_GEMV(16, NACC_, RPI_);  \
+  } while (0)
+  if (nacc == 1 && p.rows_per_instr == 1)
+    SHAINET_LAUNCH_GEMV_T(1, 1);
+  else if (nacc == 1)
+    SHAINET_LAUNCH_GEMV_T(1, 4);
+  else if (p.rows_per_instr == 1)
+    SHAINET_LAUNCH_GEMV_T(2, 1);
   else
-    SHAINET_LAUNCH_GEMV(16);
+    SHAINET_LAUNCH_GEMV_T(2, 4);
+#undef SHAINET_LAUNCH_GEMV_T
 #undef SHAINET_LAUNCH_GEMV
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  const int total = T * N / 4;
-  hipLaunchKernelGGL(gemv_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, partials, y,
-                     total, p.splits);
   return hipGetLastError();
 }
 

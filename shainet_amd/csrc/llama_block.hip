@@ -36,12 +36,12 @@ struct shainet_llama_attn {
   std::vector<float> rope_freqs, q_norm, k_norm, b_q, b_k, b_v;
   bool has_rope_freqs = false, has_q_norm = false, has_k_norm = false, has_bq = false, has_bk = false, has_bv = false;
   bool params_dirty = true;  // setters may run after construction (hf_loader.cr:319-373)
-  float *w_q = nullptr, *w_k = nullptr, *w_v = nullptr, *w_o = nullptr;  // device, [in, out]
+  float *w_qkv = nullptr, *w_o = nullptr;  // device, [in, out]; w_q | w_k | w_v side by side in one matrix
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
   int cache_len = 0;  // @cache_len
   Projector proj;
-  DevF x, q, k, v, attn, out;
+  DevF x, qkv, attn, out;
 };
 
 namespace {
@@ -85,9 +85,12 @@ void set_vec(std::vector<float> &v, bool &has, const float *src, int n) {
 }
 
 // attention_cached_cpu (llama_block.cr:246-299) with x and out on the device,
-// asynchronous on the layer's stream.
-int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out) {
-  if (!l->w_q) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
+// asynchronous on the layer's stream.  pre: an RMSNorm to apply to x on its way
+// into the projections; residual: rows to add to the result of the output
+// projection (both are what LlamaBlock#forward_cached does around attention).
+int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out, const Fused &pre = Fused(),
+                        const float *residual = nullptr) {
+  if (!l->w_qkv) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);
   if (rc) return rc;
   const int total_len = l->cache_len + T;
@@ -96,18 +99,23 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     rc = shainet_kv_cache_reserve(l->cache, total_len > 2 * cap ? total_len : 2 * cap);
     if (rc) return rc;
   }
-  const size_t qd = (size_t)T * l->q_dim, kd = (size_t)T * l->kv_dim;
-  if (!l->q.reserve(qd) || !l->k.reserve(kd) || !l->v.reserve(kd) || !l->attn.reserve(qd))
+  const int wide = l->q_dim + 2 * l->kv_dim;
+  if (!l->qkv.reserve((size_t)T * wide) || !l->attn.reserve((size_t)T * l->q_dim))
     return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
-  if ((rc = l->proj.project(x, l->w_q, l->q.p, T, l->d_model, l->q_dim, stream))) return rc;   // llama_block.cr:253
-  if ((rc = l->proj.project(x, l->w_k, l->k.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 254
-  if ((rc = l->proj.project(x, l->w_v, l->v.p, T, l->d_model, l->kv_dim, stream))) return rc;  // 255
-  rc = shainet_attn_forward(l->ctx, l->cache, nullptr, &T, 1, l->q.p, l->k.p, l->v.p, l->attn.p,
-                            SHAINET_HIP_MEM_DEVICE);  // 256-296
+  // q_full, k_new, v_new (llama_block.cr:253-255) as the three column blocks of one product
+  if ((rc = l->proj.project(x, l->d_model, l->w_qkv, l->qkv.p, T, l->d_model, wide, stream, pre))) return rc;
+  rc = shainet_attn_forward_strided(l->ctx, l->cache, nullptr, &T, 1, l->qkv.p, l->qkv.p + l->q_dim,
+                                    l->qkv.p + l->q_dim + l->kv_dim, wide, wide, wide, l->attn.p,
+                                    SHAINET_HIP_MEM_DEVICE);  // 256-296
   if (rc) return rc;
   l->cache_len = total_len;
-  return l->proj.project(l->attn.p, l->w_o, out, T, l->q_dim, l->d_model, stream);  // 298
+  Fused post;
+  if (residual) {
+    post.epilogue = kGemvResidual;
+    post.res = residual;
+  }
+  return l->proj.project(l->attn.p, l->q_dim, l->w_o, out, T, l->q_dim, l->d_model, stream, post);  // 298
 }
 
 }  // namespace
@@ -145,9 +153,9 @@ int shainet_llama_attn_destroy(shainet_llama_attn *l) {
   if (!l) return SHAINET_HIP_OK;
   drop_context(l);
   l->proj.release();
-  for (float *p : {l->w_q, l->w_k, l->w_v, l->w_o})
+  for (float *p : {l->w_qkv, l->w_o})
     if (p) (void)hipFree(p);
-  for (DevF *b : {&l->x, &l->q, &l->k, &l->v, &l->attn, &l->out}) b->release();
+  for (DevF *b : {&l->x, &l->qkv, &l->attn, &l->out}) b->release();
   delete l;
   return SHAINET_HIP_OK;
 }
@@ -183,9 +191,9 @@ int shainet_llama_attn_set_weights(shainet_llama_attn *l, const float *w_q, cons
                                    const float *w_o) {
   if (!l || !w_q || !w_k || !w_v || !w_o) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
-  int rc = upload_floats(&l->w_q, w_q, (size_t)l->d_model * l->q_dim);
-  if (!rc) rc = upload_floats(&l->w_k, w_k, (size_t)l->d_model * l->kv_dim);
-  if (!rc) rc = upload_floats(&l->w_v, w_v, (size_t)l->d_model * l->kv_dim);
+  const float *mats[3] = {w_q, w_k, w_v};
+  const int widths[3] = {l->q_dim, l->kv_dim, l->kv_dim};
+  int rc = upload_side_by_side(&l->w_qkv, mats, widths, 3, l->d_model);
   if (!rc) rc = upload_floats(&l->w_o, w_o, (size_t)l->q_dim * l->d_model);
   return rc;
 }
@@ -200,7 +208,7 @@ int shainet_llama_attn_cache_len(const shainet_llama_attn *l) { return l ? l->ca
 
 int shainet_llama_attn_forward_cached(shainet_llama_attn *l, const float *x, int new_tokens, float *out) {
   if (!l || !x || !out || new_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
-  if (!l->w_q) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
+  if (!l->w_qkv) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);  // raises what add_bias! / apply_head_rmsnorm! raise (llama_block.cr:587, 618)
   if (rc) return rc;
   const size_t xd = (size_t)new_tokens * l->d_model;
@@ -226,7 +234,7 @@ struct shainet_llama_block {
   double eps = 1e-6;                                // RMSNorm eps of @norm1 / @norm2 (llama_block.cr:93-94)
   float *norm1 = nullptr, *norm2 = nullptr;         // device gamma [d_model]; null = ones (rms_norm.cr:10)
   float *gate_up = nullptr, *down = nullptr;        // device [d_model, 2*ff] (gate | up) and [ff, d_model]
-  DevF x, normed, attn_out, h, gu, hidden, ff, out;
+  DevF x, h, hidden, out;
 };
 
 namespace {
@@ -239,24 +247,26 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
   if (rc) return rc;
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
   const int d = b->d_model, ff = b->ff_hidden;
-  const size_t xd = (size_t)T * d;
-  if (!b->normed.reserve(xd) || !b->attn_out.reserve(xd) || !b->h.reserve(xd) || !b->gu.reserve((size_t)T * 2 * ff) ||
-      !b->hidden.reserve((size_t)T * ff) || !b->ff.reserve(xd))
+  if (!b->h.reserve((size_t)T * d) || !b->hidden.reserve((size_t)T * ff))
     return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-  hipError_t e = launch_rmsnorm(x, b->norm1, b->normed.p, T, d, b->eps, stream);  // normed = @norm1.forward(x)
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("rmsnorm launch: ") + hipGetErrorString(e));
-  if ((rc = attn_forward_device(l, b->normed.p, T, b->attn_out.p))) return rc;    // attn = attention_cached_cpu(normed)
-  e = launch_add(x, b->attn_out.p, b->h.p, (long long)xd, stream);                // h = x + attn
-  if (e == hipSuccess) e = launch_rmsnorm(b->h.p, b->norm2, b->normed.p, T, d, b->eps, stream);  // normed2
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("block launch: ") + hipGetErrorString(e));
-  // ff_out = @ffn.forward(normed2): gate and up in one product against [d, 2*ff]
-  if ((rc = l->proj.project(b->normed.p, b->gate_up, b->gu.p, T, d, 2 * ff, stream))) return rc;
-  e = launch_swiglu_act(b->gu.p, b->hidden.p, T, ff, stream);
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("swiglu launch: ") + hipGetErrorString(e));
-  if ((rc = l->proj.project(b->hidden.p, b->down, b->ff.p, T, ff, d, stream))) return rc;
-  e = launch_add(b->h.p, b->ff.p, out, (long long)xd, stream);                     // h + ff_out
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("add launch: ") + hipGetErrorString(e));
-  return SHAINET_HIP_OK;
+  // h = x + attention_cached_cpu(@norm1.forward(x))
+  Fused n1;
+  n1.norm = true;
+  n1.gamma = b->norm1;
+  n1.eps = b->eps;
+  if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x))) return rc;
+  // hidden = silu(normed2 * gate_proj) * (normed2 * up_proj), normed2 = @norm2.forward(h)
+  Fused gate;
+  gate.norm = true;
+  gate.gamma = b->norm2;
+  gate.eps = b->eps;
+  gate.epilogue = kGemvSwiglu;
+  if ((rc = l->proj.project(b->h.p, d, b->gate_up, b->hidden.p, T, d, ff, stream, gate))) return rc;
+  // out = h + hidden * down_proj
+  Fused down;
+  down.epilogue = kGemvResidual;
+  down.res = b->h.p;
+  return l->proj.project(b->hidden.p, ff, b->down, out, T, ff, d, stream, down);
 }
 
 }  // namespace
@@ -264,6 +274,17 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
 // used by the model (llama_model.hip)
 int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
   return block_forward_device(b, x, T, out);
+}
+// Forget the cached rows past `len` (generation that ran ahead of a stop token).
+int shainet_llama_block_truncate(shainet_llama_block *b, int len) {
+  shainet_llama_attn *l = b->attn;
+  if (len < 0 || len > l->cache_len) return fail(SHAINET_HIP_ERR_ARGUMENT, "truncate beyond the cached length");
+  if (l->cache) {
+    int rc = shainet_kv_cache_truncate(l->cache, 0, len);
+    if (rc) return rc;
+  }
+  l->cache_len = len;
+  return SHAINET_HIP_OK;
 }
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream) {
   int rc = ensure_context(b->attn);
@@ -300,7 +321,7 @@ int shainet_llama_block_destroy(shainet_llama_block *b) {
   shainet_llama_attn_destroy(b->attn);
   for (float *p : {b->norm1, b->norm2, b->gate_up, b->down})
     if (p) (void)hipFree(p);
-  for (DevF *f : {&b->x, &b->normed, &b->attn_out, &b->h, &b->gu, &b->hidden, &b->ff, &b->out}) f->release();
+  for (DevF *f : {&b->x, &b->h, &b->hidden, &b->out}) f->release();
   delete b;
   return SHAINET_HIP_OK;
 }
@@ -327,7 +348,9 @@ int shainet_llama_block_set_norms(shainet_llama_block *b, const float *norm1, co
 int shainet_llama_block_set_ffn(shainet_llama_block *b, const float *gate, const float *up, const float *down) {
   if (!b || !gate || !up || !down) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
-  int rc = upload_side_by_side(&b->gate_up, gate, b->ff_hidden, up, b->ff_hidden, b->d_model);
+  const float *mats[2] = {gate, up};
+  const int widths[2] = {b->ff_hidden, b->ff_hidden};
+  int rc = upload_side_by_side(&b->gate_up, mats, widths, 2, b->d_model);
   if (!rc) rc = upload_floats(&b->down, down, (size_t)b->ff_hidden * b->d_model);
   return rc;
 }

@@ -5,6 +5,13 @@
 
 #include <string>
 
+#include "../../include/shainet_hip_attn.h"
+
+// capi.hip: shainet_attn_forward with the rows of q, k and v at given strides
+int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids,
+                                 const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
+                                 long long q_stride, long long k_stride, long long v_stride, float *out, int mem);
+
 namespace shainet {
 
 struct DevF {
@@ -14,21 +21,37 @@ struct DevF {
   void release();
 };
 
-// y[T,N] = x[T,K] * W[K,N], all row-major on the device: a hand-written split
-// GEMV for up to 16 rows (decode), rocBLAS SGEMM (the counterpart of the
-// reference's cuBLAS SGEMM, cuda.cr:237-247) for more.
+// What rides along with a projection y = x W.
+struct Fused {
+  int epilogue = 0;            // kGemvPlain, kGemvResidual (y = res + x W) or kGemvSwiglu (W = gate | up, [K, 2N])
+  const float *res = nullptr;  // [T, N]
+  bool norm = false;           // RMSNorm the rows of x first
+  const float *gamma = nullptr;
+  double eps = 0.0;
+};
+
+// y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows
+// (decode) run as one hand-written split GEMV with the norm and the epilogue
+// inside; more rows run as rocBLAS SGEMM (the counterpart of the reference's
+// cuBLAS SGEMM, cuda.cr:237-247) between the separate norm and epilogue kernels.
 struct Projector {
   void *blas = nullptr;
-  DevF scratch;
+  DevF scratch, normed, wide;
+  int *counters = nullptr;
+  size_t counters_cap = 0;
   // returns a SHAINET_HIP_* status; the message is left for shainet_hip_last_error
-  int project(const float *x, const float *w, float *y, int T, int K, int N, hipStream_t stream);
+  int project(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
+              const Fused &f = Fused());
   void release();
+
+ private:
+  int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
 };
 
 // Replace *dst (device, hipMalloc'ed or null) by a copy of n host floats.
 int upload_floats(float **dst, const float *src, size_t n);
-// Two host matrices [rows, n_a] and [rows, n_b] side by side into one device matrix [rows, n_a + n_b].
-int upload_side_by_side(float **dst, const float *a, int n_a, const float *b, int n_b, int rows);
+// Host matrices [rows, n_i] side by side into one device matrix [rows, sum n_i].
+int upload_side_by_side(float **dst, const float *const *mats, const int *widths, int count, int rows);
 
 int llama_fail(int code, const std::string &msg);
 

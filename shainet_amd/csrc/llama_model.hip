@@ -20,6 +20,7 @@ using namespace shainet;
 // llama_block.hip
 int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out);
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream);
+int shainet_llama_block_truncate(shainet_llama_block *b, int len);
 
 struct shainet_llama_model {
   int vocab = 0, d_model = 0;
@@ -32,7 +33,7 @@ struct shainet_llama_model {
   float *lm_bias = nullptr;     // device [vocab] or null
   hipStream_t stream = nullptr;
   Projector proj;
-  DevF act[2], normed, logits;
+  DevF act[2], logits;
   int *d_tokens = nullptr;
   size_t d_tokens_cap = 0;
   bool have_logits = false;
@@ -41,6 +42,7 @@ struct shainet_llama_model {
   size_t topk_scratch_cap = 0;
   int *d_ids = nullptr;    // kMaxTopK ids, then the count
   float *d_vals = nullptr;
+  int *d_gen = nullptr;    // generated ids of one chunk of shainet_llama_model_generate_greedy
 };
 
 namespace {
@@ -89,6 +91,35 @@ int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *v
   return SHAINET_HIP_OK;
 }
 
+// Network#run on token ids that already sit in device memory; asynchronous.
+int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T) {
+  const int d = m->d_model;
+  if (!m->act[0].reserve((size_t)T * d) || !m->act[1].reserve((size_t)T * d) || !m->logits.reserve((size_t)m->vocab))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  m->have_logits = false;
+  hipError_t e = launch_embed(m->embedding, d_tokens, m->act[0].p, T, d, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
+  int cur = 0, rc;
+  for (shainet_llama_block *b : m->blocks) {
+    if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
+    if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
+    cur ^= 1;
+  }
+  // the final norm runs over every row in the reference; only the last one is used afterwards
+  const float *last = m->act[cur].p + (size_t)(T - 1) * d;
+  Fused fin;
+  fin.norm = m->has_final_norm;
+  fin.gamma = m->final_norm;
+  fin.eps = m->eps;
+  if ((rc = m->proj.project(last, d, m->lm_head, m->logits.p, 1, d, m->vocab, m->stream, fin))) return rc;
+  if (m->lm_bias) {
+    e = launch_add_bias_row(m->logits.p, m->lm_bias, m->vocab, m->stream);
+    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("bias launch: ") + hipGetErrorString(e));
+  }
+  m->have_logits = true;
+  return SHAINET_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -123,9 +154,10 @@ int shainet_llama_model_destroy(shainet_llama_model *m) {
     if (p) (void)hipFree(p);
   if (m->d_tokens) (void)hipFree(m->d_tokens);
   if (m->d_ids) (void)hipFree(m->d_ids);
+  if (m->d_gen) (void)hipFree(m->d_gen);
   if (m->topk_scratch) (void)hipFree(m->topk_scratch);
   m->proj.release();
-  for (DevF *f : {&m->act[0], &m->act[1], &m->normed, &m->logits}) f->release();
+  for (DevF *f : {&m->act[0], &m->act[1], &m->logits}) f->release();
   if (m->stream) (void)hipStreamDestroy(m->stream);
   delete m;
   return SHAINET_HIP_OK;
@@ -183,42 +215,69 @@ int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tok
     if (tokens[i] < 0 || tokens[i] >= m->vocab) return fail(SHAINET_HIP_ERR_ARGUMENT, "token id outside the vocabulary");
   if (!m->stream && hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamCreate failed");
-  const int T = n_tokens, d = m->d_model;
-  int rc = reserve_ints(&m->d_tokens, &m->d_tokens_cap, (size_t)T);
+  int rc = reserve_ints(&m->d_tokens, &m->d_tokens_cap, (size_t)n_tokens);
   if (rc) return rc;
-  if (!m->act[0].reserve((size_t)T * d) || !m->act[1].reserve((size_t)T * d) || !m->normed.reserve((size_t)T * d) ||
-      !m->logits.reserve((size_t)m->vocab))
-    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   m->have_logits = false;
   // pageable source: the copy has left the host buffer when the call returns
-  if (hipMemcpyAsync(m->d_tokens, tokens, (size_t)T * sizeof(int), hipMemcpyHostToDevice, m->stream) != hipSuccess)
+  if (hipMemcpyAsync(m->d_tokens, tokens, (size_t)n_tokens * sizeof(int), hipMemcpyHostToDevice, m->stream) !=
+      hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(tokens) failed");
-  hipError_t e = launch_embed(m->embedding, m->d_tokens, m->act[0].p, T, d, m->stream);
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
-  int cur = 0;
-  for (shainet_llama_block *b : m->blocks) {
-    if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
-    if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
-    cur ^= 1;
-  }
-  // the final norm runs over every row in the reference; only the last one is used afterwards
-  const float *last = m->act[cur].p + (size_t)(T - 1) * d;
-  if (m->has_final_norm) {
-    e = launch_rmsnorm(last, m->final_norm, m->normed.p, 1, d, m->eps, m->stream);
-    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("rmsnorm launch: ") + hipGetErrorString(e));
-    last = m->normed.p;
-  }
-  if ((rc = m->proj.project(last, m->lm_head, m->logits.p, 1, d, m->vocab, m->stream))) return rc;
-  if (m->lm_bias) {
-    e = launch_add_bias_row(m->logits.p, m->lm_bias, m->vocab, m->stream);
-    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("bias launch: ") + hipGetErrorString(e));
-  }
-  m->have_logits = true;
+  if ((rc = run_device_tokens(m, m->d_tokens, n_tokens))) return rc;
   if (logits) {
     if (hipMemcpyAsync(logits, m->logits.p, (size_t)m->vocab * sizeof(float), hipMemcpyDeviceToHost, m->stream) !=
             hipSuccess ||
         hipStreamSynchronize(m->stream) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
+  }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_generate_greedy(shainet_llama_model *m, int max_tokens, const int *stop_ids, int n_stop,
+                                        int *out, int *n_out) {
+  if (!m || !out || !n_out || max_tokens < 0 || (n_stop > 0 && !stop_ids))
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
+  *n_out = 0;
+  if (!m->have_logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "no logits: call shainet_llama_model_run first");
+  constexpr int kChunk = 16;  // steps queued between two looks at the generated ids
+  if (!m->d_gen && hipMalloc((void **)&m->d_gen, kChunk * sizeof(int)) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  const size_t need = topk_scratch_bytes(m->vocab, 1);
+  if (need > m->topk_scratch_cap) {
+    if (m->topk_scratch) (void)hipFree(m->topk_scratch);
+    m->topk_scratch = nullptr;
+    m->topk_scratch_cap = 0;
+    if (hipMalloc(&m->topk_scratch, need) != hipSuccess) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+    m->topk_scratch_cap = need;
+  }
+  int host_ids[kChunk];
+  while (*n_out < max_tokens) {
+    const int steps = max_tokens - *n_out < kChunk ? max_tokens - *n_out : kChunk;
+    const int len0 = shainet_llama_model_cache_len(m);
+    for (int i = 0; i < steps; ++i) {
+      // best_id = Sampler.greedy(logits) into d_gen[i]; then net.run([best_id]) reading it from there
+      hipError_t e = launch_topk(m->logits.p, m->vocab, 1, true, m->topk_scratch, m->d_gen + i, nullptr, nullptr,
+                                 m->stream, 0);
+      if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("argmax launch: ") + hipGetErrorString(e));
+      int rc = run_device_tokens(m, m->d_gen + i, 1);
+      if (rc) return rc;
+    }
+    if (hipMemcpyAsync(host_ids, m->d_gen, steps * sizeof(int), hipMemcpyDeviceToHost, m->stream) != hipSuccess ||
+        hipStreamSynchronize(m->stream) != hipSuccess)
+      return fail(SHAINET_HIP_ERR_RUNTIME, "copying the generated ids back failed");
+    for (int i = 0; i < steps; ++i) {
+      bool stop = false;
+      for (int j = 0; j < n_stop; ++j) stop = stop || host_ids[i] == stop_ids[j];
+      if (stop) {
+        // the device ran ahead: the caches keep the rows of the i tokens before the stop token
+        for (shainet_llama_block *b : m->blocks) {
+          int rc = shainet_llama_block_truncate(b, len0 + i);
+          if (rc) return rc;
+        }
+        m->have_logits = false;  // the row on the device belongs to a later position
+        return SHAINET_HIP_OK;
+      }
+      out[(*n_out)++] = host_ids[i];
+    }
   }
   return SHAINET_HIP_OK;
 }

@@ -38,10 +38,10 @@ __device__ __forceinline__ RowRef locate_row(const PrepArgs &a, const SeqTable &
     while (s + 1 < st.n_seqs && token >= st.tok_off[s + 1]) ++s;
   }
   rr.pos = st.start_pos[s] + (token - st.tok_off[s]);
-  const int hd = sh.hd, q_dim = sh.H * hd, kv_dim = sh.KV * hd;
+  const int hd = sh.hd, q_dim = sh.H * hd;
   rr.rotate = true;
   if (r < sh.H) {
-    rr.src = a.q + (long long)token * q_dim + r * hd;
+    rr.src = a.q + (long long)token * a.q_stride + r * hd;
     rr.bias = a.b_q ? a.b_q + r * hd : nullptr;
     rr.w = a.q_norm;
     rr.dst = a.q_rot + (long long)token * q_dim + r * hd;
@@ -50,13 +50,13 @@ __device__ __forceinline__ RowRef locate_row(const PrepArgs &a, const SeqTable &
     const int c = is_v ? r - sh.H - sh.KV : r - sh.H;
     const long long row = (long long)st.slot[s] * sh.seq_stride + ((long long)c * sh.cap + rr.pos) * hd;
     if (is_v) {
-      rr.src = a.v + (long long)token * kv_dim + c * hd;
+      rr.src = a.v + (long long)token * a.v_stride + c * hd;
       rr.bias = a.b_v ? a.b_v + c * hd : nullptr;
       rr.w = nullptr;
       rr.dst = a.vc + row;
       rr.rotate = false;
     } else {
-      rr.src = a.k + (long long)token * kv_dim + c * hd;
+      rr.src = a.k + (long long)token * a.k_stride + c * hd;
       rr.bias = a.b_k ? a.b_k + c * hd : nullptr;
       rr.w = a.k_norm;
       rr.dst = a.kc + row;
@@ -192,9 +192,9 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
   for (int t0 = 0; t0 < total_tokens; t0 += 65535) {
     const int nt = total_tokens - t0 < 65535 ? total_tokens - t0 : 65535;
     PrepArgs b = a;
-    b.q += (long long)t0 * sh.H * sh.hd;
-    b.k += (long long)t0 * sh.KV * sh.hd;
-    b.v += (long long)t0 * sh.KV * sh.hd;
+    b.q += (long long)t0 * a.q_stride;
+    b.k += (long long)t0 * a.k_stride;
+    b.v += (long long)t0 * a.v_stride;
     b.q_rot += (long long)t0 * sh.H * sh.hd;
     SeqTable sub = st;
     if (t0) {  // the kernel indexes tokens from 0: shift the prefix sums

@@ -107,6 +107,8 @@ _SIGNATURES = {
     "shainet_llama_model_read_logits": (C.c_int, [C.c_void_p, _f32p]),
     "shainet_llama_model_write_logits": (C.c_int, [C.c_void_p, _f32p]),
     "shainet_llama_model_greedy": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
+    "shainet_llama_model_generate_greedy": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.c_int,
+                                                      C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "shainet_llama_model_repetition_penalty": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_double]),
     "shainet_llama_model_topk": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), _f32p, C.POINTER(C.c_int)]),
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
@@ -564,6 +566,19 @@ class LlamaModel:
 
     def sync(self):
         _check(lib().shainet_llama_model_sync(self._h))
+
+    def generate_greedy(self, max_tokens, stop_ids=()):
+        """The greedy generation loop on the device, from the logits of the last `run`: returns
+        the generated ids (without the stop id that ended it, if any)."""
+        import numpy as np
+
+        out = np.empty(max(max_tokens, 1), np.int32)
+        stop = np.ascontiguousarray(list(stop_ids), np.int32)
+        n = C.c_int()
+        _check(lib().shainet_llama_model_generate_greedy(
+            self._h, max_tokens, stop.ctypes.data_as(C.POINTER(C.c_int)) if stop.size else None, stop.size,
+            out.ctypes.data_as(C.POINTER(C.c_int)), C.byref(n)))
+        return [int(t) for t in out[:n.value]]
 
     def logits(self):
         import numpy as np

@@ -163,6 +163,35 @@ def test_tiny_llama_greedy_generation_matches_oracle(hip):
     rm.assert_close(m.logits(), ol, ATOL, RTOL, "logits after 12 generated tokens")
 
 
+def test_generate_greedy_on_device_matches_the_step_loop(hip):
+    m, w = _tiny_model(hip)
+    toks = [1, 42, 100]
+    m.run(toks, want_logits=False)
+    want = []
+    for _ in range(40):                       # two and a half chunks of queued steps
+        nxt = hip.Sampler.greedy(m)
+        want.append(nxt)
+        m.run([nxt], want_logits=False)
+    last = m.logits()
+    m.clear_cache()
+    m.run(toks, want_logits=False)
+    got = m.generate_greedy(40)
+    assert got == want and m.cache_len == 3 + 40
+    np.testing.assert_array_equal(m.logits(), last)
+    # a stop id: generation ends before it, the caches keep only the rows before it
+    stop_at = 21
+    assert want[stop_at] not in want[:stop_at], "pick another position: the stop id must not occur earlier"
+    m.clear_cache()
+    m.run(toks, want_logits=False)
+    got = m.generate_greedy(40, stop_ids=[want[stop_at], 31999])
+    assert got == want[:stop_at] and m.cache_len == 3 + stop_at
+    # the model continues correctly from there
+    m.run([want[stop_at]], want_logits=False)
+    assert hip.Sampler.greedy(m) == want[stop_at + 1]
+    with pytest.raises(hip.ArgumentError):
+        hip.LlamaModel(16, 8, 1, 1, 8).generate_greedy(3)     # no logits yet
+
+
 # ---- the sampler on the device ---------------------------------------------------------------
 @pytest.fixture(scope="module")
 def sampler_model(hip):
