@@ -267,6 +267,46 @@ int shainet_llama_model_repetition_penalty(shainet_llama_model *model, const int
  * *count = entries written (< k when fewer are eligible) */
 int shainet_llama_model_topk(shainet_llama_model *model, int k, int *ids, float *vals, int *count);
 
+/* ---- SafeTensors and the HuggingFace loader --------------------------------------
+ *
+ * SHAInet::SafeTensors::File / ShardedFile (src/shainet/safetensors.cr) over
+ * memory-mapped files, host only.  `path` is a .safetensors file, or a model
+ * directory holding model.safetensors or model.safetensors.index.json
+ * (HFLoader.open_safetensors, hf_loader.cr:14-26). */
+typedef struct shainet_safetensors shainet_safetensors;
+int shainet_safetensors_open(const char *path, shainet_safetensors **out);
+int shainet_safetensors_close(shainet_safetensors *st);
+int shainet_safetensors_count(const shainet_safetensors *st);               /* tensor_names.size */
+const char *shainet_safetensors_name(const shainet_safetensors *st, int i); /* tensor_names[i] */
+int shainet_safetensors_has(const shainet_safetensors *st, const char *name);  /* has_tensor? : 1 or 0 */
+/* dtype as the file spells it ("F32", "BF16", ...), up to 8 shape entries, bytes of data; any of the
+ * four outputs may be null */
+int shainet_safetensors_info(const shainet_safetensors *st, const char *name, char dtype[8], long long shape[8],
+                             int *ndim, long long *nbytes);
+/* read_f32 (safetensors.cr:90-124): F32, F16, BF16 and F64 tensors as fp32; n must be the element count */
+int shainet_safetensors_read_f32(const shainet_safetensors *st, const char *name, float *out, long long n);
+
+/* config.json of a LLaMA-family model as HFLoader.load_llama_config reads it (hf_loader.cr:199-233);
+ * head_dim 0 = not given (d_model / num_heads), num_experts 0 = dense. */
+typedef struct {
+  char model_type[32];
+  int vocab_size, hidden_size, num_attention_heads, num_hidden_layers, intermediate_size, num_key_value_heads;
+  int head_dim, tie_word_embeddings, num_experts;
+  double rms_norm_eps, rope_theta;
+  int rope_llama3; /* rope_scaling of type "llama3" present */
+  double rope_factor, rope_low_freq_factor, rope_high_freq_factor;
+  int rope_original_max_position_embeddings;
+} shainet_hf_llama_config;
+int shainet_hf_read_llama_config(const char *model_dir, shainet_hf_llama_config *cfg);
+/* HFLoader.compute_rope_freqs (hf_loader.cr:235-265): writes head_dim / 2 inverse frequencies and
+ * returns that count, returns 0 when the config has no llama3 scaling (the block then uses
+ * theta^(-2i/d)), or minus a status code.  n = room in out. */
+int shainet_hf_rope_freqs(const shainet_hf_llama_config *cfg, float *out, int n);
+/* HFLoader.load_llama (hf_loader.cr:277-412) onto the device, dense models only ("llama",
+ * "mistral", "qwen2", "qwen3"): every tensor goes to the GPU in its stored type and is converted
+ * to fp32 and transposed to [in, out] there.  The model is ready for shainet_llama_model_run. */
+int shainet_hf_load_llama(const char *model_dir, shainet_llama_model **out);
+
 /* Kernel timing for benchmarks: while enabled, every shainet_attn_forward call
  * brackets its attention kernel (the split-K decode kernel, the MFMA prefill
  * kernel or the generic kernel; not the prep or combine kernels) with HIP events

@@ -275,6 +275,25 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
 int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
   return block_forward_device(b, x, T, out);
 }
+int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out) {
+  shainet_llama_attn *l = b->attn;
+  const size_t d = (size_t)b->d_model, ff = (size_t)b->ff_hidden;
+  struct Want {
+    float **p;
+    size_t n;
+  } wants[] = {{&l->w_qkv, d * (size_t)(l->q_dim + 2 * l->kv_dim)}, {&l->w_o, (size_t)l->q_dim * d},
+               {&b->gate_up, d * 2 * ff},                            {&b->down, ff * d},
+               {&b->norm1, d},                                       {&b->norm2, d}};
+  for (const Want &w : wants)
+    if (!*w.p && hipMalloc((void **)w.p, w.n * sizeof(float)) != hipSuccess) {
+      *w.p = nullptr;
+      return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+    }
+  *out = LlamaBlockBuffers{l->w_qkv, l->w_o, b->gate_up, b->down, b->norm1, b->norm2,
+                           b->d_model, l->q_dim, l->kv_dim, b->ff_hidden};
+  return SHAINET_HIP_OK;
+}
+
 // Forget the cached rows past `len` (generation that ran ahead of a stop token).
 int shainet_llama_block_truncate(shainet_llama_block *b, int len) {
   shainet_llama_attn *l = b->attn;

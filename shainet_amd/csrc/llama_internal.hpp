@@ -12,6 +12,18 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
                                  const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                                  long long q_stride, long long k_stride, long long v_stride, float *out, int mem);
 
+// Device weight buffers of a block / a model, allocated on first request, for a loader
+// that fills them on the device (llama_block.hip, llama_model.hip).
+struct LlamaBlockBuffers {
+  float *w_qkv, *w_o, *gate_up, *down, *norm1, *norm2;
+  int d_model, q_dim, kv_dim, ff_hidden;
+};
+int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out);
+struct LlamaModelBuffers {
+  float *embedding, *final_norm, *lm_head;
+};
+int shainet_llama_model_buffers(shainet_llama_model *m, LlamaModelBuffers *out);
+
 namespace shainet {
 
 struct DevF {

@@ -49,6 +49,29 @@ namespace {
 
 int fail(int code, const std::string &msg) { return llama_fail(code, msg); }
 
+}  // namespace
+
+int shainet_llama_model_buffers(shainet_llama_model *m, LlamaModelBuffers *out) {
+  struct Want {
+    float **p;
+    size_t n;
+  } wants[] = {{&m->embedding, (size_t)m->vocab * m->d_model},
+               {&m->final_norm, (size_t)m->d_model},
+               {&m->lm_head, (size_t)m->d_model * m->vocab}};
+  for (const Want &w : wants)
+    if (!*w.p && hipMalloc((void **)w.p, w.n * sizeof(float)) != hipSuccess) {
+      *w.p = nullptr;
+      return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+    }
+  m->has_final_norm = true;
+  if (m->lm_bias) (void)hipFree(m->lm_bias);  // the loader's output bias is all zeros (hf_loader.cr:404)
+  m->lm_bias = nullptr;
+  *out = LlamaModelBuffers{m->embedding, m->final_norm, m->lm_head};
+  return SHAINET_HIP_OK;
+}
+
+namespace {
+
 int reserve_ints(int **p, size_t *cap, size_t n) {
   if (n <= *cap) return SHAINET_HIP_OK;
   size_t want = *cap ? *cap : 256;

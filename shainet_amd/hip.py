@@ -92,6 +92,17 @@ _SIGNATURES = {
     "shainet_llama_block_clear_cache": (C.c_int, [C.c_void_p]),
     "shainet_llama_block_cache_len": (C.c_int, [C.c_void_p]),
     "shainet_llama_block_forward_cached": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]),
+    "shainet_safetensors_open": (C.c_int, [C.c_char_p, C.POINTER(C.c_void_p)]),
+    "shainet_safetensors_close": (C.c_int, [C.c_void_p]),
+    "shainet_safetensors_count": (C.c_int, [C.c_void_p]),
+    "shainet_safetensors_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "shainet_safetensors_has": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "shainet_safetensors_info": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_longlong),
+                                           C.POINTER(C.c_int), C.POINTER(C.c_longlong)]),
+    "shainet_safetensors_read_f32": (C.c_int, [C.c_void_p, C.c_char_p, _f32p, C.c_longlong]),
+    "shainet_hf_read_llama_config": (C.c_int, [C.c_char_p, C.c_void_p]),
+    "shainet_hf_rope_freqs": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
+    "shainet_hf_load_llama": (C.c_int, [C.c_char_p, C.POINTER(C.c_void_p)]),
     "shainet_llama_model_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
                                              C.c_int, C.c_int, C.c_double, C.c_double]),
     "shainet_llama_model_destroy": (C.c_int, [C.c_void_p]),
@@ -503,11 +514,14 @@ class LlamaModel:
     `Sampler`."""
 
     def __init__(self, vocab, d_model, n_layers, num_heads, ff_hidden, eps=1e-6, rope_theta=10000.0,
-                 num_kv_heads=None, head_dim=None):
+                 num_kv_heads=None, head_dim=None, _loaded=None):
         num_kv_heads = num_heads if num_kv_heads is None else num_kv_heads
         self._h = C.c_void_p()
-        _check(lib().shainet_llama_model_create(C.byref(self._h), vocab, d_model, n_layers, num_heads, num_kv_heads,
-                                                head_dim or 0, ff_hidden, eps, rope_theta))
+        if _loaded is not None:  # a handle HFLoader.load_llama built
+            self._h = _loaded
+        else:
+            _check(lib().shainet_llama_model_create(C.byref(self._h), vocab, d_model, n_layers, num_heads,
+                                                    num_kv_heads, head_dim or 0, ff_hidden, eps, rope_theta))
         self.vocab, self.d_model, self.n_layers = vocab, d_model, n_layers
         self.blocks = [LlamaBlock(d_model, num_heads, ff_hidden, eps, rope_theta, num_kv_heads, head_dim,
                                   _borrowed=lib().shainet_llama_model_block(self._h, i)) for i in range(n_layers)]
@@ -657,3 +671,95 @@ class Sampler:
                 best = int(ids[i])
                 break
         return best
+
+
+class SafeTensors:
+    """SHAInet::SafeTensors::File / ShardedFile (safetensors.cr): a .safetensors file, or a model
+    directory with model.safetensors or model.safetensors.index.json.  Host only."""
+
+    def __init__(self, path):
+        self._h = C.c_void_p()
+        _check(lib().shainet_safetensors_open(os.fsencode(path), C.byref(self._h)))
+
+    def close(self):
+        if getattr(self, "_h", None) and lib is not None:
+            lib().shainet_safetensors_close(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def tensor_names(self):
+        L = lib()
+        return [L.shainet_safetensors_name(self._h, i).decode() for i in range(L.shainet_safetensors_count(self._h))]
+
+    def has_tensor(self, name):
+        return bool(lib().shainet_safetensors_has(self._h, name.encode()))
+
+    def info(self, name):
+        dt = C.create_string_buffer(8)
+        shape = (C.c_longlong * 8)()
+        nd, nb = C.c_int(), C.c_longlong()
+        _check(lib().shainet_safetensors_info(self._h, name.encode(), dt, shape, C.byref(nd), C.byref(nb)))
+        return dt.value.decode(), [int(shape[i]) for i in range(nd.value)], int(nb.value)
+
+    def read_f32(self, name):
+        import numpy as np
+
+        dtype, shape, nbytes = self.info(name)
+        size = {"F16": 2, "BF16": 2, "F32": 4, "F64": 8}.get(dtype, 1)
+        out = np.empty(nbytes // size, np.float32)
+        _check(lib().shainet_safetensors_read_f32(self._h, name.encode(), out.ctypes.data_as(_f32p), out.size))
+        return out
+
+    def read_matrix(self, name):
+        """read_matrix (safetensors.cr:161-187): 1-D tensors come back as one row."""
+        _, shape, _ = self.info(name)
+        if len(shape) > 2:
+            raise ArgumentError(f"Cannot read tensor '{name}' with {len(shape)}D shape as matrix")
+        rows = 1 if len(shape) < 2 else shape[0]
+        return self.read_f32(name).reshape(rows, -1)
+
+
+class _HFLlamaConfig(C.Structure):
+    _fields_ = [("model_type", C.c_char * 32), ("vocab_size", C.c_int), ("hidden_size", C.c_int),
+                ("num_attention_heads", C.c_int), ("num_hidden_layers", C.c_int), ("intermediate_size", C.c_int),
+                ("num_key_value_heads", C.c_int), ("head_dim", C.c_int), ("tie_word_embeddings", C.c_int),
+                ("num_experts", C.c_int), ("rms_norm_eps", C.c_double), ("rope_theta", C.c_double),
+                ("rope_llama3", C.c_int), ("rope_factor", C.c_double), ("rope_low_freq_factor", C.c_double),
+                ("rope_high_freq_factor", C.c_double), ("rope_original_max_position_embeddings", C.c_int)]
+
+
+class HFLoader:
+    """HFLoader (hf_loader.cr) for LLaMA-family models: config.json, llama3 RoPE frequencies and
+    load_llama onto the device."""
+
+    @staticmethod
+    def load_llama_config(model_dir):
+        cfg = _HFLlamaConfig()
+        _check(lib().shainet_hf_read_llama_config(os.fsencode(model_dir), C.byref(cfg)))
+        d = {name: getattr(cfg, name) for name, _ in _HFLlamaConfig._fields_}
+        d["model_type"] = d["model_type"].decode()
+        d["_struct"] = cfg
+        return d
+
+    @staticmethod
+    def compute_rope_freqs(config):
+        """Array of head_dim/2 inverse frequencies, or None when the config has no llama3 scaling."""
+        import numpy as np
+
+        cfg = config["_struct"]
+        hd = cfg.head_dim or cfg.hidden_size // max(cfg.num_attention_heads, 1)
+        out = np.empty(max(hd // 2, 1), np.float32)
+        n = lib().shainet_hf_rope_freqs(C.byref(cfg), out.ctypes.data_as(_f32p), hd // 2)
+        if n < 0:
+            _check(-n)
+        return out[:n] if n > 0 else None
+
+    @staticmethod
+    def load_llama(model_dir):
+        cfg = HFLoader.load_llama_config(model_dir)
+        h = C.c_void_p()
+        _check(lib().shainet_hf_load_llama(os.fsencode(model_dir), C.byref(h)))
+        return LlamaModel(cfg["vocab_size"], cfg["hidden_size"], cfg["num_hidden_layers"], cfg["num_attention_heads"],
+                          cfg["intermediate_size"], cfg["rms_norm_eps"], cfg["rope_theta"],
+                          cfg["num_key_value_heads"], cfg["head_dim"] or None, _loaded=h)

@@ -268,3 +268,128 @@ def test_device_repetition_penalty_and_sample_match_oracle(hip, sampler_model):
     for r in (0.0, 0.03, 0.25, 0.5, 0.77, 0.999999):
         s.rng = Fixed(r)
         assert s.sample(m) == orc.sample(want, 40, 0.6, r)
+
+
+# ---- HFLoader.load_llama on the device --------------------------------------------------------
+def test_load_llama_tiny_llama_matches_fixture_and_setter_built_model(hip, golden_dir):
+    # spec/llama_loader_spec.cr: load tiny-llama, run [1, 42, 100]
+    d = np.load(os.path.join(golden_dir, "tiny_llama_logits.npz"))
+    m = hip.HFLoader.load_llama(tinyllama.DIR)
+    assert (m.vocab, m.d_model, m.n_layers) == (32000, 16, 2)
+    got = m.run(d["tokens_t3"])
+    assert got.shape == (32000,) and np.isfinite(got).all()
+    assert np.abs(got - d["logits_t3"]).max() < 1e-5
+    ref, _ = _tiny_model(hip)                       # the same weights through the setters
+    np.testing.assert_array_equal(got, ref.run(d["tokens_t3"]))
+    np.testing.assert_array_equal(m.run(d["tokens_t4"][3:]), ref.run(d["tokens_t4"][3:]))
+
+
+def _write_st(path, tensors):
+    import json
+    import struct
+
+    header, blob = {}, b""
+    for name, (dtype, arr) in tensors.items():
+        raw = arr.tobytes()
+        header[name] = {"dtype": dtype, "shape": list(arr.shape), "data_offsets": [len(blob), len(blob) + len(raw)]}
+        blob += raw
+    h = json.dumps(header).encode()
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(h)) + h + blob)
+
+
+def test_load_llama_bf16_f16_sharded_qwen_style(hip, tmp_path):
+    import json
+
+    r = np.random.default_rng(9)
+    V, d, L, H, KV, hd, ff = 512, 128, 2, 4, 2, 64, 256     # explicit head_dim: q_dim 256 != d_model
+    cfg = {"model_type": "qwen3", "vocab_size": V, "hidden_size": d, "num_attention_heads": H,
+           "num_hidden_layers": L, "intermediate_size": ff, "rms_norm_eps": 1e-6, "num_key_value_heads": KV,
+           "head_dim": hd, "rope_parameters": {"rope_theta": 1e6}, "tie_word_embeddings": True,
+           "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                            "original_max_position_embeddings": 64}}
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+
+    def bf16(a):   # stored as bf16 bit patterns; value = those bits << 16
+        bits = (np.asarray(a, np.float32).view(np.uint32) >> 16).astype("<u2")
+        return ("BF16", bits), (bits.astype(np.uint32) << 16).view(np.float32)
+
+    def f16(a):
+        # value as SafeTensors::File#f16_to_f32 computes it (safetensors.cr:189-218): IEEE for normal
+        # halves; for a subnormal half the exponent field is 127 + e, e = -1 - (shifts to normalise)
+        h = np.asarray(a, np.float32).astype("<f2")
+        bits = h.view(np.uint16).astype(np.uint32)
+        value = h.astype(np.float32)
+        sub = ((bits >> 10) & 0x1F == 0) & (bits & 0x3FF != 0)
+        for i in np.flatnonzero(sub.reshape(-1)):
+            b = int(bits.reshape(-1)[i])
+            mant, e = b & 0x3FF, -1
+            while mant & 0x400 == 0:
+                mant, e = mant << 1, e - 1
+            w = ((b >> 15) << 31) | ((127 + e) << 23) | ((mant & 0x3FF) << 13)
+            value.reshape(-1)[i] = np.array([w], np.uint32).view(np.float32)[0]
+        return ("F16", h), value
+
+    shards, weight_map, vals = [{}, {}], {}, {}
+
+    def put(name, arr, enc, shard):
+        stored, value = enc(arr)
+        shards[shard][name] = stored
+        weight_map[name] = f"model-0000{shard + 1}-of-00002.safetensors"
+        vals[name] = value
+
+    put("model.embed_tokens.weight", 0.05 * r.standard_normal((V, d)), bf16, 0)
+    put("model.norm.weight", 1 + 0.1 * r.standard_normal(d), f16, 1)
+    for li in range(L):
+        p = f"model.layers.{li}."
+        enc = bf16 if li == 0 else f16
+        put(p + "self_attn.q_proj.weight", 0.05 * r.standard_normal((H * hd, d)), enc, li)
+        put(p + "self_attn.k_proj.weight", 0.05 * r.standard_normal((KV * hd, d)), enc, li)
+        put(p + "self_attn.v_proj.weight", 0.05 * r.standard_normal((KV * hd, d)), enc, 1 - li)
+        put(p + "self_attn.o_proj.weight", 0.05 * r.standard_normal((d, H * hd)), enc, li)
+        put(p + "mlp.gate_proj.weight", 0.05 * r.standard_normal((ff, d)), enc, li)
+        put(p + "mlp.up_proj.weight", 0.05 * r.standard_normal((ff, d)), enc, 1 - li)
+        put(p + "mlp.down_proj.weight", 0.05 * r.standard_normal((d, ff)), enc, li)
+        put(p + "input_layernorm.weight", 1 + 0.1 * r.standard_normal(d), enc, li)
+        put(p + "post_attention_layernorm.weight", 1 + 0.1 * r.standard_normal(d), enc, li)
+        put(p + "self_attn.q_norm.weight", 1 + 0.1 * r.standard_normal(hd), enc, li)
+        put(p + "self_attn.k_norm.weight", 1 + 0.1 * r.standard_normal(hd), enc, li)
+        put(p + "self_attn.q_proj.bias", 0.2 * r.standard_normal(H * hd), enc, li)
+        put(p + "self_attn.k_proj.bias", 0.2 * r.standard_normal(KV * hd), enc, li)
+        put(p + "self_attn.v_proj.bias", 0.2 * r.standard_normal(KV * hd), enc, li)
+    for i, sh in enumerate(shards):
+        _write_st(tmp_path / f"model-0000{i + 1}-of-00002.safetensors", sh)
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+
+    m = hip.HFLoader.load_llama(str(tmp_path))
+    c = hip.HFLoader.load_llama_config(str(tmp_path))
+    freqs = hip.HFLoader.compute_rope_freqs(c)
+    assert freqs is not None and freqs.shape == (hd // 2,)
+    ref = hip.LlamaModel(V, d, L, H, ff, eps=1e-6, rope_theta=1e6, num_kv_heads=KV, head_dim=hd)
+    ref.set_embedding(vals["model.embed_tokens.weight"])
+    ref.set_final_norm(vals["model.norm.weight"])
+    ref.set_lm_head(np.ascontiguousarray(vals["model.embed_tokens.weight"].T))   # tied
+    T = lambda n: np.ascontiguousarray(vals[n].T)
+    for li, b in enumerate(ref.blocks):
+        p = f"model.layers.{li}."
+        b.set_rope(1e6, freqs)
+        b.set_weights(T(p + "self_attn.q_proj.weight"), T(p + "self_attn.k_proj.weight"),
+                      T(p + "self_attn.v_proj.weight"), T(p + "self_attn.o_proj.weight"))
+        b.set_ffn(T(p + "mlp.gate_proj.weight"), T(p + "mlp.up_proj.weight"), T(p + "mlp.down_proj.weight"))
+        b.set_norms(vals[p + "input_layernorm.weight"], vals[p + "post_attention_layernorm.weight"])
+        b.set_qk_norm(vals[p + "self_attn.q_norm.weight"], vals[p + "self_attn.k_norm.weight"])
+        b.set_bias(vals[p + "self_attn.q_proj.bias"], vals[p + "self_attn.k_proj.bias"],
+                   vals[p + "self_attn.v_proj.bias"])
+    toks = list(r.integers(0, V, 21))
+    np.testing.assert_array_equal(m.run(toks), ref.run(toks))           # prefill (library GEMM)
+    for t in (3, 77):
+        np.testing.assert_array_equal(m.run([t]), ref.run([t]))         # decode (fused GEMV)
+    # a missing tensor and an unsupported model type are reported, not half-loaded
+    del weight_map["model.norm.weight"]
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+    with pytest.raises(hip.ArgumentError, match="model.norm.weight"):
+        hip.HFLoader.load_llama(str(tmp_path))
+    cfg["model_type"] = "qwen3_moe"
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    with pytest.raises(hip.ArgumentError, match="mixture-of-experts"):
+        hip.HFLoader.load_llama(str(tmp_path))
