@@ -55,6 +55,7 @@ struct DecodePlan {
   int n_wgs;
   int n_slots;  // partial slots: workgroup index + pair index is unique per segment
 };
+// wg_target: 0 = default
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 

@@ -96,8 +96,8 @@ __device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last
   }
 }
 
-template <int HD>
-__global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__restrict__ q_rot,
+template <int HD, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(const float *__restrict__ q_rot,
                                                                const float *__restrict__ kc,
                                                                const float *__restrict__ vc,
                                                                float *__restrict__ out, float *part_o,
@@ -106,9 +106,11 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
                                                                int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
-  __shared__ __attribute__((aligned(1024))) char k_lds[4][2][C::TILE_BYTES];
-  extern __shared__ float merge_lds[];  // [4][g][HD] O, [4][g] max, [4][g] sum
+  __shared__ __attribute__((aligned(1024))) char k_lds[NW][2][C::TILE_BYTES];
+  // after its last tile a wavefront parks its O rows [g][HD] in its own K tile area
+  __shared__ float sm_m[NW][16], sm_l[NW][16];  // per wavefront and head: running max, sum
   __shared__ bool last_flag;
+  constexpr int WAVE_LDS_FLOATS = 2 * C::TILE_BYTES / 4;  // floats between two wavefronts' areas
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, j = lane >> 4;
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         qr[4 * i + 3] = x.w;
       }
     }
-    for (int it = 0; tile < tile1; tile += 4, ++it) {
+    for (int it = 0; tile < tile1; tile += NW, ++it) {
       const int kb = tile * 16;
       char *buf = my_lds + (it & 1) * C::TILE_BYTES;
       // everything issued so far (this tile's K copy and V loads) has landed:
@@ -169,9 +171,9 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
       for (int r = 0; r < 4; ++r)
 #pragma unroll
         for (int u = 0; u < C::NVU; ++u) v_cur[r][u] = v_next[r][u];
-      if (tile + 4 < tile1) {
-        issue_k_tile<HD>(kbase, kb + 64, L - 1, my_lds + ((it + 1) & 1) * C::TILE_BYTES, lane);
-        load_v_tile<HD>(vbase, kb + 64, L - 1, col, j, v_next);
+      if (tile + NW < tile1) {
+        issue_k_tile<HD>(kbase, kb + 16 * NW, L - 1, my_lds + ((it + 1) & 1) * C::TILE_BYTES, lane);
+        load_v_tile<HD>(vbase, kb + 16 * NW, L - 1, col, j, v_next);
       }
 
       f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -210,39 +212,37 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         }
     }
 
-    // merge the four wavefronts through LDS
+    // merge the wavefronts through LDS: each one's tiles are consumed, so its K tile
+    // area is free to hold its O rows
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    float *sm_o = merge_lds;
-    float *sm_m = merge_lds + 4 * g * HD;
-    float *sm_l = sm_m + 4 * g;
-    __syncthreads();  // the previous segment's readers are done with merge_lds
+    float *sm_o = (float *)&k_lds[0][0][0];
     if (col < g) {
-      float *dst = sm_o + (wave * g + col) * HD;
+      float *dst = sm_o + wave * WAVE_LDS_FLOATS + col * HD;
 #pragma unroll
       for (int i = 0; i < NT; ++i)
 #pragma unroll
         for (int r = 0; r < 4; ++r) dst[64 * (i >> 2) + 4 * (4 * j + r) + (i & 3)] = o[i][r];
       if (j == 0) {
-        sm_m[wave * g + col] = m;
-        sm_l[wave * g + col] = l;
+        sm_m[wave][col] = m;
+        sm_l[wave][col] = l;
       }
     }
     __syncthreads();
     const bool whole_pair = tile0 == 0 && tile1 == n_s;
     const int pair = s * sh.KV + kvh;
     const int slot = blockIdx.x + pair;  // unique: both terms only grow along the tile stream
-    for (int idx = threadIdx.x; idx < g * HD; idx += 256) {
+    for (int idx = threadIdx.x; idx < g * HD; idx += 64 * NW) {
       const int cc = idx / HD, d = idx - cc * HD;
-      float mm = sm_m[cc];
+      float mm = sm_m[0][cc];
 #pragma unroll
-      for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w * g + cc]);
+      for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w][cc]);
       float acc = 0.f, ls = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const float f = fast_exp2((sm_m[w * g + cc] - mm) * c);  // 0 for a wavefront that saw no tile
-        acc += f * sm_o[(w * g + cc) * HD + d];
-        ls += f * sm_l[w * g + cc];
+      for (int w = 0; w < NW; ++w) {
+        const float f = fast_exp2((sm_m[w][cc] - mm) * c);  // 0 for a wavefront that saw no tile
+        acc += f * sm_o[w * WAVE_LDS_FLOATS + cc * HD + d];
+        ls += f * sm_l[w][cc];
       }
       if (whole_pair) {
         out[((long long)token * sh.H + kvh * g + cc) * HD + d] = acc / ls;
@@ -255,16 +255,17 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         }
       }
     }
+    // Every wavefront is done with the O rows parked in LDS (the next segment's K
+    // tiles land there).  Partials are written through to device-coherent memory
+    // (coherent_store); the barrier also waits for this workgroup's stores to be
+    // acknowledged before its arrival is counted.
+    __syncthreads();
     if (!whole_pair) {
       // The last workgroup to deliver a partial of this pair merges them all.  The
       // counter returns to zero for the next launch.
       const int a = st.work_off[s] + kvh * n_s;  // the pair's tiles are [a, a + n_s)
       const int w_lo = a / tiles_per_wg, w_hi = (a + n_s - 1) / tiles_per_wg;
       const int n_part = w_hi - w_lo + 1;
-      // Partials are written through to device-coherent memory (coherent_store);
-      // the barrier waits for this workgroup's stores to be acknowledged before
-      // its arrival is counted.
-      __syncthreads();
       if (threadIdx.x == 0) {
         const int old = atomicAdd(&pair_count[pair], 1);
         last_flag = old == n_part - 1;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
         constexpr int GROUPS = 64 / LPR;  // partials handled side by side
         const int d4 = lane % LPR, grp = lane / LPR;
         const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
-        for (int cc = wave; cc < g; cc += 4) {
+        for (int cc = wave; cc < g; cc += NW) {
           const long long first = base + cc;
           float mm = -INFINITY;
           for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
@@ -325,6 +326,7 @@ __global__ __launch_bounds__(256, 2) void decode_splitk_kernel(const float *__re
 }
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kDecodeWaves = 4;  // wavefronts per workgroup (eight measured no better)
 
 }  // namespace
 
@@ -334,10 +336,14 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   for (int s = 0; s < st.n_seqs; ++s)
     st.work_off[s + 1] = st.work_off[s] + sh.KV * ((st.start_pos[s] + 1 + 15) / 16);
   p.total_tiles = st.work_off[st.n_seqs];
-  if (wg_target < 1) wg_target = 512;  // two workgroups on each of the 256 compute units
-  // at least four tiles (one per wavefront) per workgroup
+  // One workgroup on each of the 256 compute units.  Its four wavefronts keep 64 KiB
+  // of K and V in flight, 16 MiB over the chip, which saturates HBM; twice as many
+  // workgroups only double the partials to merge and the arrivals at each pair's
+  // counter (measured: 4 to 10 % slower from batch 1 x 4096 to batch 4 x 32768).
+  if (wg_target < 1) wg_target = 256;
+  // at least one tile per wavefront
   int q = (p.total_tiles + wg_target - 1) / wg_target;
-  if (q < 4) q = 4;
+  if (q < kDecodeWaves) q = kDecodeWaves;
   p.tiles_per_wg = q;
   p.n_wgs = (p.total_tiles + q - 1) / q;
   p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
@@ -360,15 +366,14 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   float *part_o = d.partials;
   float *part_ml = d.partials + (size_t)p.n_slots * sh.g * sh.hd;
   const float c = scale * kLog2e;
-  const size_t smem = (size_t)(4 * sh.g * sh.hd + 8 * sh.g) * sizeof(float);
   if (before) (void)hipEventRecord(before, stream);
-  dim3 grid((unsigned)p.n_wgs), block(256);
+  dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
-    hipLaunchKernelGGL(decode_splitk_kernel<64>, grid, block, smem, stream, d.q_rot, d.kc, d.vc, d.out, part_o,
-                       part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, d.q_rot, d.kc, d.vc, d.out,
+                       part_o, part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
   else
-    hipLaunchKernelGGL(decode_splitk_kernel<128>, grid, block, smem, stream, d.q_rot, d.kc, d.vc, d.out, part_o,
-                       part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, d.q_rot, d.kc, d.vc, d.out,
+                       part_o, part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
   hipError_t e = hipGetLastError();
   if (after) (void)hipEventRecord(after, stream);
   return e;
