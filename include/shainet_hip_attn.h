@@ -186,6 +186,9 @@ int shainet_llama_attn_clear_cache(shainet_llama_attn *layer);
 int shainet_llama_attn_cache_len(const shainet_llama_attn *layer);
 /* attention_cached_cpu (246-299): x and out are host [new_tokens, d_model]; synchronous. */
 int shainet_llama_attn_forward_cached(shainet_llama_attn *layer, const float *x, int new_tokens, float *out);
+/* attention_full_cpu (209-243), the no-cache path of LlamaBlock#forward: the same arithmetic from
+ * position 0 over the seq_len rows of x alone; @cache_len and the cached rows are left as they are. */
+int shainet_llama_attn_forward_full(shainet_llama_attn *layer, const float *x, int seq_len, float *out);
 
 /* ---- the whole block ---------------------------------------------------------
  *
@@ -215,6 +218,8 @@ int shainet_llama_block_cache_len(const shainet_llama_block *block);
  * SHAINET_HIP_MEM_DEVICE: device pointers, asynchronous on the block's stream. */
 int shainet_llama_block_forward_cached(shainet_llama_block *block, const float *x, int new_tokens, float *out,
                                        int mem);
+/* LlamaBlock#forward (179-186): the whole sequence without the cache (Network#run with use_kv_cache off). */
+int shainet_llama_block_forward(shainet_llama_block *block, const float *x, int seq_len, float *out, int mem);
 
 /* ---- the model around the blocks ----------------------------------------------
  *

@@ -39,6 +39,7 @@ struct shainet_llama_attn {
   float *w_qkv = nullptr, *w_o = nullptr;  // device, [in, out]; w_q | w_k | w_v side by side in one matrix
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
+  shainet_kv_cache *scratch_cache = nullptr;  // rows of a no-cache forward call; empty between calls
   int cache_len = 0;  // @cache_len
   Projector proj;
   DevF x, qkv, attn, out;
@@ -49,6 +50,8 @@ namespace {
 constexpr int kInitialCapacity = 256;  // llama_block.cr:500
 
 void drop_context(shainet_llama_attn *l) {
+  if (l->scratch_cache) shainet_kv_cache_destroy(l->scratch_cache);
+  l->scratch_cache = nullptr;
   if (l->cache) shainet_kv_cache_destroy(l->cache);
   if (l->ctx) shainet_attn_destroy(l->ctx);
   l->cache = nullptr;
@@ -88,15 +91,26 @@ void set_vec(std::vector<float> &v, bool &has, const float *src, int n) {
 // asynchronous on the layer's stream.  pre: an RMSNorm to apply to x on its way
 // into the projections; residual: rows to add to the result of the output
 // projection (both are what LlamaBlock#forward_cached does around attention).
+//
+// no_cache: attention_full_cpu (209-243) instead: the same arithmetic from
+// position 0 over the rows of this call alone; they go through a scratch cache
+// that is empty again afterwards, and the block's own cache is not touched.
 int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out, const Fused &pre = Fused(),
-                        const float *residual = nullptr) {
+                        const float *residual = nullptr, bool no_cache = false) {
   if (!l->w_qkv) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);
   if (rc) return rc;
-  const int total_len = l->cache_len + T;
-  const int cap = shainet_kv_cache_capacity(l->cache);
+  shainet_kv_cache *cache = l->cache;
+  if (no_cache) {
+    if (!l->scratch_cache && (rc = shainet_kv_cache_create(&l->scratch_cache, l->ctx, 1, T > kInitialCapacity ? T : kInitialCapacity)))
+      return rc;
+    cache = l->scratch_cache;
+    if ((rc = shainet_kv_cache_clear(cache, -1))) return rc;
+  }
+  const int total_len = (no_cache ? 0 : l->cache_len) + T;
+  const int cap = shainet_kv_cache_capacity(cache);
   if (total_len > cap) {  // ensure_gpu_cache! (llama_block.cr:497-520): grow by doubling, contents stay on the device
-    rc = shainet_kv_cache_reserve(l->cache, total_len > 2 * cap ? total_len : 2 * cap);
+    rc = shainet_kv_cache_reserve(cache, total_len > 2 * cap ? total_len : 2 * cap);
     if (rc) return rc;
   }
   const int wide = l->q_dim + 2 * l->kv_dim;
@@ -105,11 +119,15 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
   // q_full, k_new, v_new (llama_block.cr:253-255) as the three column blocks of one product
   if ((rc = l->proj.project(x, l->d_model, l->w_qkv, l->qkv.p, T, l->d_model, wide, stream, pre))) return rc;
-  rc = shainet_attn_forward_strided(l->ctx, l->cache, nullptr, &T, 1, l->qkv.p, l->qkv.p + l->q_dim,
+  rc = shainet_attn_forward_strided(l->ctx, cache, nullptr, &T, 1, l->qkv.p, l->qkv.p + l->q_dim,
                                     l->qkv.p + l->q_dim + l->kv_dim, wide, wide, wide, l->attn.p,
                                     SHAINET_HIP_MEM_DEVICE);  // 256-296
   if (rc) return rc;
-  l->cache_len = total_len;
+  if (no_cache) {
+    if ((rc = shainet_kv_cache_clear(cache, -1))) return rc;
+  } else {
+    l->cache_len = total_len;
+  }
   Fused post;
   if (residual) {
     post.epilogue = kGemvResidual;
@@ -206,7 +224,17 @@ int shainet_llama_attn_clear_cache(shainet_llama_attn *l) {
 
 int shainet_llama_attn_cache_len(const shainet_llama_attn *l) { return l ? l->cache_len : -1; }
 
+static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_tokens, float *out, bool no_cache);
+
 int shainet_llama_attn_forward_cached(shainet_llama_attn *l, const float *x, int new_tokens, float *out) {
+  return attn_forward_host(l, x, new_tokens, out, false);
+}
+
+int shainet_llama_attn_forward_full(shainet_llama_attn *l, const float *x, int seq_len, float *out) {
+  return attn_forward_host(l, x, seq_len, out, true);
+}
+
+static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_tokens, float *out, bool no_cache) {
   if (!l || !x || !out || new_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
   if (!l->w_qkv) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);  // raises what add_bias! / apply_head_rmsnorm! raise (llama_block.cr:587, 618)
@@ -216,7 +244,7 @@ int shainet_llama_attn_forward_cached(shainet_llama_attn *l, const float *x, int
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
   if (hipMemcpyAsync(l->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
-  if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p))) return rc;
+  if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p, Fused(), nullptr, no_cache))) return rc;
   if (hipMemcpyAsync(out, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
@@ -240,7 +268,7 @@ struct shainet_llama_block {
 namespace {
 
 // x and out on the device; asynchronous on the block's stream.
-int block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
+int block_forward_device(shainet_llama_block *b, const float *x, int T, float *out, bool no_cache = false) {
   if (!b->gate_up || !b->down) return fail(SHAINET_HIP_ERR_ARGUMENT, "feed-forward weights not set");
   shainet_llama_attn *l = b->attn;
   int rc = ensure_context(l);
@@ -254,7 +282,7 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
   n1.norm = true;
   n1.gamma = b->norm1;
   n1.eps = b->eps;
-  if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x))) return rc;
+  if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x, no_cache))) return rc;
   // hidden = silu(normed2 * gate_proj) * (normed2 * up_proj), normed2 = @norm2.forward(h)
   Fused gate;
   gate.norm = true;
@@ -381,11 +409,21 @@ int shainet_llama_block_clear_cache(shainet_llama_block *b) {
 
 int shainet_llama_block_cache_len(const shainet_llama_block *b) { return b ? b->attn->cache_len : -1; }
 
+static int block_forward_any(shainet_llama_block *b, const float *x, int new_tokens, float *out, int mem, bool no_cache);
+
 int shainet_llama_block_forward_cached(shainet_llama_block *b, const float *x, int new_tokens, float *out, int mem) {
+  return block_forward_any(b, x, new_tokens, out, mem, false);
+}
+
+int shainet_llama_block_forward(shainet_llama_block *b, const float *x, int seq_len, float *out, int mem) {
+  return block_forward_any(b, x, seq_len, out, mem, true);
+}
+
+static int block_forward_any(shainet_llama_block *b, const float *x, int new_tokens, float *out, int mem, bool no_cache) {
   if (!b || !x || !out || new_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
   if (mem != SHAINET_HIP_MEM_HOST && mem != SHAINET_HIP_MEM_DEVICE)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "mem must be SHAINET_HIP_MEM_HOST or SHAINET_HIP_MEM_DEVICE");
-  if (mem == SHAINET_HIP_MEM_DEVICE) return block_forward_device(b, x, new_tokens, out);
+  if (mem == SHAINET_HIP_MEM_DEVICE) return block_forward_device(b, x, new_tokens, out, no_cache);
   int rc = ensure_context(b->attn);
   if (rc) return rc;
   const size_t xd = (size_t)new_tokens * b->d_model;
@@ -393,7 +431,7 @@ int shainet_llama_block_forward_cached(shainet_llama_block *b, const float *x, i
   hipStream_t stream = (hipStream_t)shainet_attn_stream(b->attn->ctx);
   if (hipMemcpyAsync(b->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
-  if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p))) return rc;
+  if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p, no_cache))) return rc;
   if (hipMemcpyAsync(out, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");

@@ -83,6 +83,8 @@ _SIGNATURES = {
     "shainet_llama_attn_clear_cache": (C.c_int, [C.c_void_p]),
     "shainet_llama_attn_cache_len": (C.c_int, [C.c_void_p]),
     "shainet_llama_attn_forward_cached": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p]),
+    "shainet_llama_attn_forward_full": (C.c_int, [C.c_void_p, _f32p, C.c_int, _f32p]),
+    "shainet_llama_block_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]),
     "shainet_llama_block_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_double,
                                              C.c_double, C.c_int, C.c_int]),
     "shainet_llama_block_destroy": (C.c_int, [C.c_void_p]),
@@ -484,27 +486,42 @@ class LlamaBlock:
                                                        out.ctypes.data_as(_f32p)))
         return out
 
-    def forward_cached(self, x, out=None):
+    def attention_full(self, x):
+        """attention_full_cpu(x): the no-cache path; the cache is left as it is."""
+        import numpy as np
+
+        x = np.ascontiguousarray(x, np.float32)
+        if x.ndim != 2 or x.shape[1] != self.d_model:
+            raise ArgumentError(f"x must be [T, {self.d_model}]")
+        out = np.empty_like(x)
+        _check(lib().shainet_llama_attn_forward_full(self._h, x.ctypes.data_as(_f32p), x.shape[0],
+                                                     out.ctypes.data_as(_f32p)))
+        return out
+
+    def forward(self, x):
+        """LlamaBlock#forward: the whole sequence without the cache."""
+        return self.forward_cached(x, _fn="shainet_llama_block_forward")
+
+    def forward_cached(self, x, out=None, _fn="shainet_llama_block_forward_cached"):
         """LlamaBlock#forward_cached.  numpy in -> numpy out (copies, synchronous); a CUDA torch
         tensor in -> torch tensor out (device pointers, asynchronous on the block's stream)."""
         import numpy as np
 
         self._need_block()
+        call = getattr(lib(), _fn)
         if hasattr(x, "is_cuda") and x.is_cuda:
             import torch
 
             if x.dim() != 2 or x.shape[1] != self.d_model or x.dtype != torch.float32 or not x.is_contiguous():
                 raise ArgumentError(f"x must be a contiguous float32 [T, {self.d_model}] tensor")
             out = torch.empty_like(x) if out is None else out
-            _check(lib().shainet_llama_block_forward_cached(self._block, x.data_ptr(), x.shape[0], out.data_ptr(),
-                                                            MEM_DEVICE))
+            _check(call(self._block, x.data_ptr(), x.shape[0], out.data_ptr(), MEM_DEVICE))
             return out
         x = np.ascontiguousarray(x, np.float32)
         if x.ndim != 2 or x.shape[1] != self.d_model:
             raise ArgumentError(f"x must be [T, {self.d_model}]")
         out = np.empty_like(x)
-        _check(lib().shainet_llama_block_forward_cached(self._block, x.ctypes.data, x.shape[0], out.ctypes.data,
-                                                        MEM_HOST))
+        _check(call(self._block, x.ctypes.data, x.shape[0], out.ctypes.data, MEM_HOST))
         return out
 
 

@@ -87,6 +87,32 @@ def test_block_llama1b_shape_prefill_and_decode(hip):
         rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, f"decode {i}")
 
 
+@pytest.mark.parametrize("d,H,KV,hd,ff,norm,bias", [
+    (64, 8, 4, None, 96, False, False),
+    (128, 8, 2, 64, 344, True, True),
+])
+def test_block_forward_without_cache_matches_oracle(hip, d, H, KV, hd, ff, norm, bias):
+    # LlamaBlock#forward / attention_full_cpu: the no-cache path must not disturb the cache
+    blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e4, seed=d, norm=norm, bias=bias)
+    x0 = r.standard_normal((7, d)).astype(np.float32)
+    rm.assert_close(blk.forward_cached(x0), _oracle_forward(ob, p, eps, x0), ATOL, RTOL, "cached prefill")
+    for T in (1, 19, 300):                                    # 300 outgrows the scratch cache's first capacity
+        x = r.standard_normal((T, d)).astype(np.float32)
+        want = ob.forward(x, p["norm1"], p["norm2"], eps, p["gate"], p["up"], p["down"], False)
+        rm.assert_close(blk.forward(x), want, ATOL, RTOL, f"no-cache forward T={T}")
+        rm.assert_close(blk.attention_full(x), ob.attention_full(x), ATOL, RTOL, f"attention_full T={T}")
+        assert blk.cache_len == ob.cache_len == 7
+    x1 = r.standard_normal((1, d)).astype(np.float32)         # the cached path continues where it was
+    rm.assert_close(blk.forward_cached(x1), _oracle_forward(ob, p, eps, x1), ATOL, RTOL, "decode after no-cache calls")
+    # cached == full recompute on the last row (spec/rope_kv_cache_spec.cr:29-59)
+    blk.clear_cache()
+    xs = r.standard_normal((6, d)).astype(np.float32)
+    full = blk.forward(xs)
+    blk.forward_cached(xs[:5])
+    last = blk.forward_cached(xs[5:])
+    assert np.abs(last[0] - full[5]).max() < 1e-3
+
+
 def test_block_device_pointers_match_host_pointers(hip):
     import torch
 
