@@ -19,6 +19,7 @@
 #include "attn_kernels.hpp"
 
 #include <math.h>
+#include <stdlib.h>
 
 namespace shainet {
 
@@ -70,8 +71,13 @@ __device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &
   vb = st.work_off[s] - 1 - level;
 }
 
-template <int HD, bool SPLIT>
-__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__restrict__ q_rot,
+// G = 1: four wavefronts, each with 32 virtual rows, walk the key tiles together.
+// G = 2: eight wavefronts; wavefronts 4..7 own the same rows as 0..3 and take every
+// second key tile, so that each SIMD holds two wavefronts of one workgroup and the
+// vector-ALU work of one hides behind the MFMAs of the other even when a launch
+// puts a single workgroup on a compute unit.  The two halves merge through LDS.
+template <int HD, bool SPLIT, int G>
+__global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(const float *__restrict__ q_rot,
                                                               const float *__restrict__ kc,
                                                               const float *__restrict__ vc,
                                                               float *__restrict__ out,
@@ -81,9 +87,11 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   constexpr int NK4 = HD / 8;   // float4 pieces of a K row per lane
   constexpr int NT = HD / 32;   // d tiles of the output
   constexpr int KSTR = HD + 4;  // padded K row stride in LDS: conflict-free 16-byte reads down a column
-  constexpr int LD4 = HD / 32;  // float4 per thread to stage one K (or V) tile
-  __shared__ float Ks[2][32 * KSTR];
-  __shared__ float Vs[2][32 * HD];
+  constexpr int LD4 = HD / 32;  // float4 per thread to stage the G K (or V) tiles of one step
+  constexpr int NTHREADS = 256 * G;
+  constexpr int TILE4 = 32 * (HD / 4);  // float4 per tile
+  __shared__ float Ks[2][G][32 * KSTR];
+  __shared__ float Vs[2][G][32 * HD];
 
   // Workgroups are numbered so that the hardware dispatcher, which hands them out in
   // index order, starts the row blocks with the longest key ranges first; the kv
@@ -98,7 +106,9 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   locate_block(st, item, s, vb);
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
   const int L = S + T, VR = T * g;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = (threadIdx.x >> 6) & 3;  // which 32 virtual rows of the block
+  const int gidx = threadIdx.x >> 8;        // which share of the key tiles (always 0 for G = 1)
   const int n = lane & 31, j = lane >> 5;
   const int v0 = vb * 128 + wave * 32;
   const bool wave_active = v0 < VR;
@@ -139,39 +149,44 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
 
-  // Staging registers: a tile travels global memory -> registers during one
-  // iteration and registers -> LDS at the start of the next.
+  // Staging registers: the G tiles of a step (tiles kt0 + G*sp .. + G-1, one per
+  // group of wavefronts) travel global memory -> registers during one iteration and
+  // registers -> LDS at the start of the next.
   f32x4 stage_k[LD4], stage_v[LD4];
-  auto load_k = [&](int kt) {
+  auto load_k = [&](int sp) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + 256 * u;
-      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
-      stage_k[u] = *(const f32x4 *)(kbase + (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4);
+      const int idx = threadIdx.x + NTHREADS * u;
+      const int ts = idx / TILE4, rem = idx - ts * TILE4;
+      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
+      stage_k[u] = *(const f32x4 *)(kbase + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
     }
   };
-  auto load_v = [&](int kt) {
+  auto load_v = [&](int sp) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + 256 * u;
-      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
-      stage_v[u] = *(const f32x4 *)(vbase + (long long)min(kt * 32 + r, L - 1) * HD + 4 * c4);
+      const int idx = threadIdx.x + NTHREADS * u;
+      const int ts = idx / TILE4, rem = idx - ts * TILE4;
+      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
+      stage_v[u] = *(const f32x4 *)(vbase + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
     }
   };
   auto store_k = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + 256 * u;
-      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
-      *(f32x4 *)&Ks[buf][r * KSTR + 4 * c4] = stage_k[u];
+      const int idx = threadIdx.x + NTHREADS * u;
+      const int ts = idx / TILE4, rem = idx - ts * TILE4;
+      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
+      *(f32x4 *)&Ks[buf][ts][r * KSTR + 4 * c4] = stage_k[u];
     }
   };
   auto store_v = [&](int buf) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + 256 * u;
-      const int r = idx / (HD / 4), c4 = idx - r * (HD / 4);
-      *(f32x4 *)&Vs[buf][r * HD + 4 * c4] = stage_v[u];
+      const int idx = threadIdx.x + NTHREADS * u;
+      const int ts = idx / TILE4, rem = idx - ts * TILE4;
+      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
+      *(f32x4 *)&Vs[buf][ts][r * HD + 4 * c4] = stage_v[u];
     }
   };
 
@@ -183,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
     f32x16 sacc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-    const float *kl = &Ks[buf][n * KSTR + 4 * j];
+    const float *kl = &Ks[buf][gidx][n * KSTR + 4 * j];
     f32x4 kv[NK4];
 #pragma unroll
     for (int i = 0; i < PF && i < NK4; ++i) kv[i] = *(const f32x4 *)(kl + 8 * i);
@@ -200,38 +215,40 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
     return sacc;
   };
 
-  // Software pipeline over the key tiles.  Iteration kt issues the MFMAs of
-  // S^T(kt+1) before the softmax arithmetic of tile kt, so the vector ALU works in
-  // their shadow, then O^T += V^T(kt) P^T(kt).  K runs two tiles ahead of V:
-  //   LDS at the start of iteration kt:  K(kt+1) in Ks[(kt+1)&1], V(kt) in Vs[kt&1];
-  //   registers:                          K(kt+2), V(kt+1), fetched during kt-1.
-  // The iteration first parks those registers in the two LDS stages nobody reads
-  // any more (Ks[kt&1] held K(kt), Vs[(kt+1)&1] held V(kt-1); both were last
-  // read in iteration kt-1), then fetches K(kt+3) and V(kt+2).  One barrier per
-  // iteration, at its end, orders all of this.
+  // Software pipeline over the key tiles, in steps of G tiles (one per group of
+  // wavefronts; below "tile sp" is this group's tile of step sp).  Step sp issues the
+  // MFMAs of S^T(sp+1) before the softmax arithmetic of tile sp, so the vector ALU
+  // works in their shadow, then O^T += V^T(sp) P^T(sp).  K runs two steps ahead of V:
+  //   LDS at the start of step sp:  K(sp+1) in Ks[(sp+1)&1], V(sp) in Vs[sp&1];
+  //   registers:                     K(sp+2), V(sp+1), fetched during step sp-1.
+  // The step first parks those registers in the two LDS stages nobody reads any
+  // more (Ks[sp&1] held K(sp), Vs[(sp+1)&1] held V(sp-1); both were last read in
+  // step sp-1), then fetches K(sp+3) and V(sp+2).  One barrier per step, at its
+  // end, orders all of this.
+  const int n_sp = kt0 < kt1 ? (kt1 - kt0 + G - 1) / G : 0;
   f32x16 s_cur, s_next;
 #pragma unroll
   for (int r = 0; r < 16; ++r) s_cur[r] = s_next[r] = 0.f;
-  if (kt0 < kt1) {
-    load_k(kt0);
-    load_v(kt0);
-    store_k(kt0 & 1);
-    store_v(kt0 & 1);
-    if (kt0 + 1 < kt1) {
-      load_k(kt0 + 1);
-      load_v(kt0 + 1);
-      store_k((kt0 + 1) & 1);
+  if (n_sp > 0) {
+    load_k(0);
+    load_v(0);
+    store_k(0);
+    store_v(0);
+    if (n_sp > 1) {
+      load_k(1);
+      load_v(1);
+      store_k(1);
     }
   }
   __syncthreads();
-  if (kt0 + 2 < kt1) load_k(kt0 + 2);
-  if (kt0 < kt1 && kt0 * 32 <= wave_hi) s_cur = scores(kt0 & 1);
-  __syncthreads();  // iteration kt0 overwrites Ks[kt0&1]
+  if (n_sp > 2) load_k(2);
+  if (kt0 + gidx < kt1 && (kt0 + gidx) * 32 <= wave_hi) s_cur = scores(0);
+  __syncthreads();  // step 0 overwrites Ks[0]
 
   // O^T += V^T P^T of one tile; the probabilities are the registers of `p`
   auto accumulate = [&](const f32x16 &p, int buf) {
     constexpr int PF = NT == 2 ? 4 : 2;
-    const float *vl = &Vs[buf][4 * j * HD + NT * n];
+    const float *vl = &Vs[buf][gidx][4 * j * HD + NT * n];
     typedef float vrow_t __attribute__((ext_vector_type(NT)));
     vrow_t vv[16];
 #pragma unroll
@@ -249,13 +266,14 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   // tiles [0, n_interior) are visible to every row of this wavefront: no masking
   const int n_interior = wave_active ? (wave_lo + 1) / 32 : 0;
 
-  for (int kt = kt0; kt < kt1; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 2 < kt1) store_k(buf);
-    if (kt + 1 < kt1) store_v(buf ^ 1);
-    if (kt + 3 < kt1) load_k(kt + 3);
-    if (kt + 2 < kt1) load_v(kt + 2);
-    if (kt + 1 < n_interior && kt + 1 < kt1) {
+  for (int sp = 0; sp < n_sp; ++sp) {
+    const int buf = sp & 1;
+    const int kt = kt0 + G * sp + gidx, kt_next = kt + G;  // this group's tile now and in the next step
+    if (sp + 2 < n_sp) store_k(buf);
+    if (sp + 1 < n_sp) store_v(buf ^ 1);
+    if (sp + 3 < n_sp) load_k(sp + 3);
+    if (sp + 2 < n_sp) load_v(sp + 2);
+    if (kt_next < n_interior && kt_next < kt1) {
       // Hot path, one basic block: the score MFMAs of tile kt+1 and the softmax
       // arithmetic of tile kt are independent, so the scheduler can interleave them.
       s_next = scores(buf ^ 1);
@@ -281,8 +299,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
       m = mnew;
       accumulate(sacc, buf);
     } else {
-      if (kt + 1 < kt1 && (kt + 1) * 32 <= wave_hi) s_next = scores(buf ^ 1);
-      if (kt * 32 <= wave_hi) {
+      if (kt_next < kt1 && kt_next * 32 <= wave_hi) s_next = scores(buf ^ 1);
+      if (kt < kt1 && kt * 32 <= wave_hi) {
         f32x16 sacc = s_cur;
         if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
 #pragma unroll
@@ -296,8 +314,9 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
         for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float mnew = fmaxf(m, mx);
-        // a chunk that starts past a row's last visible key leaves that row at -inf
-        const float mref = SPLIT && mnew == -INFINITY ? 0.f : mnew;
+        // a key chunk (or, with two groups, the second group's first tile) that starts past
+        // a row's last visible key leaves that row at -inf
+        const float mref = (SPLIT || G == 2) && mnew == -INFINITY ? 0.f : mnew;
         const float alpha = fast_exp2((m - mref) * c);
         const float mc = mref * c;
         float psum = 0.f;
@@ -320,6 +339,33 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(const float *__res
   }
 
   l += __shfl_xor(l, 32);
+  if constexpr (G == 2) {
+    // the second group hands its (max, sum, O) to the first through the tile stages
+    // (every wavefront is past the last step's barrier: nobody reads tiles any more)
+    float *xo = &Ks[0][0][0];  // [4 row chunks][16 * NT registers][64 lanes]
+    float *xm = &Vs[0][0][0];  // [4][64] max, then [4][64] sum
+    if (gidx == 1) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) xo[((wave * NT + t) * 16 + r) * 64 + lane] = o[t][r];
+      xm[wave * 64 + lane] = m;
+      xm[256 + wave * 64 + lane] = l;
+    }
+    __syncthreads();
+    if (gidx == 1) return;
+    const float m1 = xm[wave * 64 + lane], l1 = xm[256 + wave * 64 + lane];
+    const float mnew = fmaxf(m, m1);
+    // a side that saw no visible key has max -inf: its factor is 0 (and both may be, in a key chunk)
+    const float a0 = m == -INFINITY ? 0.f : fast_exp2((m - mnew) * c);
+    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2((m1 - mnew) * c);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[t][r] = o[t][r] * a0 + xo[((wave * NT + t) * 16 + r) * 64 + lane] * a1;
+    l = l * a0 + l1 * a1;
+    m = mnew;
+  }
   if (SPLIT) {  // unnormalised partial of this key chunk: [128 virtual rows][HD], (max, sum) per row
     const long long pbase = (((long long)item * sh.KV + kvh) * ns + chunk) * 128 + wave * 32 + n;
     float *op = part_o + pbase * HD;
@@ -514,8 +560,13 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
   dim3 grid((unsigned)n_wgs);
   float *part_o = partials;
   float *part_ml = partials ? partials + (size_t)items * sh.KV * ns * 128 * sh.hd : nullptr;
-  // static LDS of the kernel: two stages of a padded K tile and a V tile
-  const size_t static_lds = (size_t)2 * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
+  // With fewer workgroups than three per compute unit everything is resident at
+  // once: run one workgroup per compute unit (below) and give it eight wavefronts,
+  // two per SIMD (G = 2).  Larger launches already have several workgroups per unit.
+  static const int groups_env = getenv("SHAINET_HIP_PREFILL_GROUPS") ? atoi(getenv("SHAINET_HIP_PREFILL_GROUPS")) : 0;
+  const int groups = groups_env == 1 || groups_env == 2 ? groups_env : (n_wgs <= 768 ? 2 : 1);
+  // static LDS of the kernel: two stages of `groups` padded K tiles and V tiles
+  const size_t static_lds = (size_t)2 * groups * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
   size_t pad = 0;
   // With fewer workgroups than three per compute unit everything is resident at
   // once and the dispatcher cannot balance the triangular work: one workgroup per
@@ -526,9 +577,15 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
     const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
     if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
   }
-#define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                     \
-  hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_>), grid, dim3(256), pad, stream, q_rot, kc, vc, out, part_o, \
-                     part_ml, st, sh, ns, c)
+#define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                    \
+  do {                                                                                                          \
+    if (groups == 2)                                                                                            \
+      hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, q_rot, kc, vc, out, \
+                         part_o, part_ml, st, sh, ns, c);                                                       \
+    else                                                                                                        \
+      hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, q_rot, kc, vc, out, \
+                         part_o, part_ml, st, sh, ns, c);                                                       \
+  } while (0)
   if (sh.hd == 64) {
     if (ns > 1)
       SHAINET_LAUNCH_PREFILL(64, true);

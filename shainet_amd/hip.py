@@ -315,6 +315,28 @@ class AttnContext:
         return out
 
 
+    def prepared(self, cache, q, k, v, new_tokens, out, seq_ids=None):
+        """A zero-argument callable that repeats this device-pointer forward call with nothing but
+        the C call in it (tight decode loops, benchmarks): the argument checks of `forward` run
+        once, here.  The tensors must stay alive and in place while the callable is used."""
+        n = len(new_tokens)
+        nt = (C.c_int * n)(*new_tokens)
+        ids = (C.c_int * n)(*seq_ids) if seq_ids is not None else None
+        rows = sum(new_tokens)
+        assert q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and out.is_contiguous()
+        assert tuple(q.shape) == (rows, self.q_dim) and tuple(k.shape) == (rows, self.kv_dim)
+        assert tuple(v.shape) == tuple(k.shape) and tuple(out.shape) == tuple(q.shape)
+        fn, h, ch = lib().shainet_attn_forward, self._h, cache._h
+        qp, kp, vp, op = (C.c_void_p(t.data_ptr()) for t in (q, k, v, out))
+
+        def call():
+            rc = fn(h, ch, ids, nt, n, qp, kp, vp, op, MEM_DEVICE)
+            if rc:
+                _check(rc)
+
+        return call
+
+
 class KVCache:
     """Device-resident fp32 KV cache: [batch][num_kv_heads][capacity][head_dim] for K and V."""
 
