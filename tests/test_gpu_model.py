@@ -77,6 +77,16 @@ def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, 
     rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, "after clear")
 
 
+def test_block_every_small_row_count(hip):
+    # 1..16 rows take the fused split GEMV (norm inside for up to 4 rows, a norm kernel first above
+    # that), 17 and more the library GEMM: every count around those switches
+    blk, ob, p, r, eps = _block_pair(hip, 256, 8, 2, 64, 512, 1e4, seed=11, norm=True, bias=True)
+    for T in (2, 4, 5, 8, 15, 16, 17, 1):
+        x = r.standard_normal((T, 256)).astype(np.float32)
+        rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, f"T={T}")
+    assert blk.cache_len == ob.cache_len == 68
+
+
 def test_block_llama1b_shape_prefill_and_decode(hip):
     # Llama-3.2-1B block: hidden 2048, 32 Q / 8 KV heads, head_dim 64, ff 8192, theta 5e5
     blk, ob, p, r, eps = _block_pair(hip, 2048, 32, 8, None, 8192, 500000.0, seed=7, wscale=0.02, eps=1e-5)
