@@ -44,10 +44,14 @@ struct Fused {
 
 // y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows
 // (decode) run as one hand-written split GEMV with the norm and the epilogue
-// inside; more rows run as rocBLAS SGEMM (the counterpart of the reference's
-// cuBLAS SGEMM, cuda.cr:237-247) between the separate norm and epilogue kernels.
+// inside; more rows run as a library SGEMM (rocBLAS or hipBLASLt by shape, the
+// counterpart of the reference's cuBLAS SGEMM, cuda.cr:237-247) between the separate
+// norm and epilogue kernels.
+struct LtState;
 struct Projector {
   void *blas = nullptr;
+  LtState *lt = nullptr;
+  bool lt_broken = false;
   DevF scratch, normed, wide;
   int *counters = nullptr;
   size_t counters_cap = 0;
@@ -58,6 +62,7 @@ struct Projector {
 
  private:
   int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
+  int gemm_lt(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
 };
 
 // Replace *dst (device, hipMalloc'ed or null) by a copy of n host floats.

@@ -87,10 +87,19 @@ def test_block_every_small_row_count(hip):
     assert blk.cache_len == ob.cache_len == 68
 
 
+def test_block_many_rows_both_library_gemms(hip):
+    # more than 16 rows: rocBLAS below 256 rows of a small weight matrix, hipBLASLt from 256 rows on
+    blk, ob, p, r, eps = _block_pair(hip, 128, 8, 2, 64, 344, 1e4, seed=5, norm=True, bias=True)
+    for T in (40, 255, 256, 300):
+        x = r.standard_normal((T, 128)).astype(np.float32)
+        rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, f"T={T}")
+    assert blk.cache_len == ob.cache_len == 851
+
+
 def test_block_llama1b_shape_prefill_and_decode(hip):
     # Llama-3.2-1B block: hidden 2048, 32 Q / 8 KV heads, head_dim 64, ff 8192, theta 5e5
     blk, ob, p, r, eps = _block_pair(hip, 2048, 32, 8, None, 8192, 500000.0, seed=7, wscale=0.02, eps=1e-5)
-    x = r.standard_normal((24, 2048)).astype(np.float32)       # rocBLAS projections (more than 16 rows)
+    x = r.standard_normal((24, 2048)).astype(np.float32)       # library GEMMs: rocBLAS (QKV, O), hipBLASLt (gate|up, down)
     rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, "prefill 24")
     for i in range(2):                                         # split GEMV projections
         x = r.standard_normal((1, 2048)).astype(np.float32)
