@@ -86,7 +86,21 @@ hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, 
 
 // y[T,N] = epilogue(norm(x)[T,K] * W[K,N]), T <= 16, N % 4 == 0: the projections of a
 // decode step with what surrounds them fused in.
-enum { kGemvPlain = 0, kGemvResidual = 1, kGemvSwiglu = 2 };
+enum { kGemvPlain = 0, kGemvResidual = 1, kGemvSwiglu = 2, kGemvQkvPrep = 3 };
+// kGemvQkvPrep: W = W_q | W_k | W_v and the product's rows never go to memory as
+// they are: each head row gets its bias, QK-norm and rotation where it is summed up
+// and lands in q_rot (query heads) or in the cache of one sequence at positions
+// start_pos + row (key heads rotated, value heads as they are), exactly as
+// launch_prep would have left it.  head_dim: a power of two, at most 128.
+struct GemvPrep {
+  const float *b_q, *b_k, *b_v;  // nullable
+  const float *q_norm, *k_norm;  // nullable, [hd]
+  double eps;
+  const float2 *rope_tab;        // [positions][hd/2] (cos, sin)
+  float *q_rot;                  // [T, H*hd]
+  float *kc, *vc;                // the sequence's cache: [KV, cap, hd]
+  int H, KV, hd, cap, start_pos;
+};
 struct GemvArgs {
   const float *x;        // [T, K], rows x_stride floats apart
   long long x_stride;
@@ -101,6 +115,7 @@ struct GemvArgs {
   int T, K, N;
   int epilogue;
   int rows_per_wave;     // filled in by launch_gemv
+  GemvPrep prep;         // kGemvQkvPrep only (y is not written then)
 };
 struct GemvPlan {
   int rows_per_instr;     // 1: 256-column tiles; 4: 64-column tiles, four rows of W per load instruction
@@ -109,7 +124,8 @@ struct GemvPlan {
   int col_tiles;
   size_t partial_floats;  // scratch the launch needs
 };
-GemvPlan plan_gemv(int T, int K, int N, int epilogue);
+// head_dim: kGemvQkvPrep only (a column tile must hold whole heads)
+GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim = 0);
 hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
 
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,

@@ -414,9 +414,12 @@ int shainet_kv_cache_create(shainet_kv_cache **out, shainet_attn_ctx *ctx, int b
   const size_t bytes = (size_t)batch * ctx->KV * capacity * ctx->hd * sizeof(float);
   hipError_t e = hipMalloc((void **)&kc->k, bytes);
   if (e == hipSuccess) e = hipMalloc((void **)&kc->v, bytes);
-  // zero-fill: rows never appended must hold finite values
-  if (e == hipSuccess) e = hipMemset(kc->k, 0, bytes);
-  if (e == hipSuccess) e = hipMemset(kc->v, 0, bytes);
+  // zero-fill: rows never appended must hold finite values.  On the context's stream and
+  // waited for: a fill on the null stream is not ordered with the kernels that append rows
+  // (the stream is non-blocking) and could wipe rows written right after this call.
+  if (e == hipSuccess) e = hipMemsetAsync(kc->k, 0, bytes, ctx->stream);
+  if (e == hipSuccess) e = hipMemsetAsync(kc->v, 0, bytes, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (e != hipSuccess) {
     int rc = hip_fail(e, "kv cache allocation");
     shainet_kv_cache_destroy(kc);
@@ -618,6 +621,52 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
     HIP_TRY(hipStreamSynchronize(c->stream));
   }
   return SHAINET_HIP_OK;
+}
+
+int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, GemvPrep *where) {
+  if (!c || !kc || kc->ctx != c || !where)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (new_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "new_tokens must be positive");
+  if ((long long)kc->len[0] + new_tokens > kc->cap)
+    return fail(SHAINET_HIP_ERR_CAPACITY, "sequence 0: %d cached + %d new rows exceed capacity %d", kc->len[0],
+                new_tokens, kc->cap);
+  int rc = ensure_rope_table(c, kc->len[0] + new_tokens);
+  if (!rc) rc = c->q_rot.reserve((size_t)new_tokens * c->H * c->hd);
+  if (rc) return rc;
+  where->b_q = c->d_bq;
+  where->b_k = c->d_bk;
+  where->b_v = c->d_bv;
+  where->q_norm = c->d_q_norm;
+  where->k_norm = c->d_k_norm;
+  where->eps = c->eps;
+  where->rope_tab = c->d_rope;
+  where->q_rot = c->q_rot.p;
+  where->kc = kc->k;
+  where->vc = kc->v;
+  where->H = c->H;
+  where->KV = c->KV;
+  where->hd = c->hd;
+  where->cap = kc->cap;
+  where->start_pos = kc->len[0];
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out) {
+  if (!c || !kc || kc->ctx != c || !out)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (new_tokens < 1 || (long long)kc->len[0] + new_tokens > kc->cap)
+    return fail(SHAINET_HIP_ERR_CAPACITY, "sequence 0: %d cached + %d new rows exceed capacity %d", kc->len[0],
+                new_tokens, kc->cap);
+  SeqTable st;
+  memset(&st, 0, sizeof st);
+  st.n_seqs = 1;
+  st.start_pos[0] = kc->len[0];
+  st.n_new[0] = new_tokens;
+  st.tok_off[1] = new_tokens;
+  Shape sh = shape_of(c, kc->cap);
+  kc->len[0] += new_tokens;
+  c->last_rows = new_tokens;
+  return run_attention(c, c->q_rot.p, kc->k, kc->v, out, st, sh, new_tokens, c->scale, c->stream, nullptr);
 }
 
 extern "C" {

@@ -12,9 +12,12 @@
 // epilogue.  Everything a decode step does around a product rides along:
 //   * prologue: RMSNorm of the x rows (rms_norm.cr:18-37, fp64 as there), so the
 //     normalised activations never go to memory;
-//   * epilogue: residual add (simple_matrix.cr:39-48) or the SwiGLU gate
-//     (swiglu_ff.cr:84-89) over a [K, 2*ff] matrix holding gate_proj | up_proj.
+//   * epilogue: residual add (simple_matrix.cr:39-48), the SwiGLU gate
+//     (swiglu_ff.cr:84-89) over a [K, 2*ff] matrix holding gate_proj | up_proj, or,
+//     for the q | k | v product, bias -> QK-norm -> RoPE -> cache append
+//     (llama_block.cr:256-286, 332-344) on each head row where it is summed up.
 #include "attn_kernels.hpp"
+#include "prep_math.hpp"
 
 #include <math.h>
 #include <stdlib.h>
@@ -47,12 +50,58 @@ __device__ __forceinline__ f32x4 apply_epilogue(int epi, f32x4 a, f32x4 b, const
   return a;
 }
 
+// One row of the q | k | v product, complete in tile[CW] (columns tile0 ...): each
+// wavefront takes whole heads of it through the arithmetic of prep_rows_kernel.
+__device__ __forceinline__ void prep_tile_row(const GemvPrep &p, const float *tile, int tile0, int cw, int t,
+                                              int wave, int lane) {
+  const int hd = p.hd, half = hd >> 1;
+  const bool active = lane < half;
+  const int i = active ? lane : 0;
+  const int pos = p.start_pos + t;
+  for (int hh = wave; hh * hd < cw; hh += 4) {
+    const int r = tile0 / hd + hh;  // head row of the token: H query, KV key, KV value heads
+    if (r >= p.H + 2 * p.KV) break;
+    float x0 = tile[hh * hd + i], x1 = tile[hh * hd + i + half];
+    const float *bias, *w = nullptr;
+    float *dst;
+    bool rotate = true;
+    if (r < p.H) {
+      bias = p.b_q ? p.b_q + r * hd : nullptr;
+      w = p.q_norm;
+      dst = p.q_rot + (long long)t * p.H * hd + r * hd;
+    } else {
+      const bool is_v = r - p.H >= p.KV;
+      const int c = is_v ? r - p.H - p.KV : r - p.H;
+      const long long row = ((long long)c * p.cap + pos) * hd;
+      bias = is_v ? (p.b_v ? p.b_v + c * hd : nullptr) : (p.b_k ? p.b_k + c * hd : nullptr);
+      w = is_v ? nullptr : p.k_norm;
+      dst = (is_v ? p.vc : p.kc) + row;
+      rotate = !is_v;
+    }
+    if (bias) {
+      x0 = x0 + bias[i];
+      x1 = x1 + bias[i + half];
+    }
+    float y0 = x0, y1 = x1;
+    if (rotate) {
+      const float w0 = w ? w[i] : 1.0f, w1 = w ? w[i + half] : 1.0f;
+      const float2 cs = p.rope_tab[(long long)pos * half + i];
+      norm_rotate_pair(x0, x1, w != nullptr, w0, w1, p.eps, hd, half, cs, y0, y1);
+    }
+    if (active) {
+      dst[i] = y0;
+      dst[i + half] = y1;
+    }
+  }
+}
+
 // NACC = 1, or 2 for the SwiGLU epilogue (gate and up accumulators).
+// PREP: the kGemvQkvPrep epilogue (NACC = 1).
 // RPI = rows of W per load instruction: 1 (a wavefront spans 256 columns) or 4
 // (16 lanes per row, 64 columns, four consecutive rows at once).  Narrow tiles give
 // a matrix with few columns enough column tiles that 16 workgroups along K
 // suffice: the arrivals at a tile's counter serialise at roughly 0.1 us each.
-template <int TT, int NACC, int RPI>
+template <int TT, int NACC, int RPI, bool PREP>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   constexpr int LPR = 64 / RPI;  // lanes across a row
   constexpr int CW = LPR * 4;    // columns per tile
@@ -60,6 +109,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   __shared__ double rms_s[TT];
   __shared__ double red_s[4];
   __shared__ bool last_flag;
+  __shared__ __align__(16) float tile_s[PREP ? 256 : 4];  // PREP: one finished row of this column tile
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int cl = lane % LPR, sub = lane / LPR;
   const int T = a.T, K = a.K, N = a.N;
@@ -161,21 +211,32 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
         acc[c][t] = (acc[c][t] + red[(0 * TT + t) * 64 + lane]) + (red[(1 * TT + t) * 64 + lane] + red[(2 * TT + t) * 64 + lane]);
     }
   }
-  if (wave == 0 && sub == 0 && have_col) {
+  const bool writer = wave == 0 && sub == 0 && have_col;
+  if (splits == 1) {
 #pragma unroll
     for (int t = 0; t < TT; ++t)
       if (t < T) {
-        if (splits == 1) {
+        if constexpr (PREP) {
+          if (writer) *(f32x4 *)(tile_s + cl * 4) = acc[0][t];
+          __syncthreads();
+          prep_tile_row(a.prep, tile_s, blockIdx.x * CW, CW, t, wave, lane);
+          __syncthreads();
+        } else if (writer) {
           const float *res = a.res ? a.res + (long long)t * N + col : nullptr;
           *(f32x4 *)(a.y + (long long)t * N + col) = apply_epilogue(a.epilogue, acc[0][t], acc[NACC - 1][t], res);
-        } else {
-#pragma unroll
-          for (int c = 0; c < NACC; ++c)
-            coherent_store4(a.partials + (((long long)blockIdx.y * T + t) * NACC + c) * N + col, acc[c][t]);
         }
       }
+    return;
   }
-  if (splits == 1) return;
+  if (writer) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+      if (t < T) {
+#pragma unroll
+        for (int c = 0; c < NACC; ++c)
+          coherent_store4(a.partials + (((long long)blockIdx.y * T + t) * NACC + c) * N + col, acc[c][t]);
+      }
+  }
 
   // ---- the last workgroup of this column tile adds the partials in a fixed order
   __syncthreads();  // the partial stores above are acknowledged before the arrival is counted
@@ -227,21 +288,29 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 #pragma unroll
     for (int c = 0; c < NACC; ++c) red[(wave * NACC + c) * 64 + lane] = part[c];
     __syncthreads();
-    if (wave == 0 && sub == 0 && have_col) {
+    if (writer) {
       f32x4 sum[NACC];
 #pragma unroll
       for (int c = 0; c < NACC; ++c)
         sum[c] = (red[(0 * NACC + c) * 64 + lane] + red[(1 * NACC + c) * 64 + lane]) +
                  (red[(2 * NACC + c) * 64 + lane] + red[(3 * NACC + c) * 64 + lane]);
-      const float *res = a.res ? a.res + (long long)t * N + col : nullptr;
-      *(f32x4 *)(a.y + (long long)t * N + col) = apply_epilogue(a.epilogue, sum[0], sum[NACC - 1], res);
+      if constexpr (PREP) {
+        *(f32x4 *)(tile_s + cl * 4) = sum[0];
+      } else {
+        const float *res = a.res ? a.res + (long long)t * N + col : nullptr;
+        *(f32x4 *)(a.y + (long long)t * N + col) = apply_epilogue(a.epilogue, sum[0], sum[NACC - 1], res);
+      }
+    }
+    if constexpr (PREP) {
+      __syncthreads();  // the row is complete in tile_s; the next round's first barrier protects it
+      prep_tile_row(a.prep, tile_s, blockIdx.x * CW, CW, t, wave, lane);
     }
   }
 }
 
 }  // namespace
 
-GemvPlan plan_gemv(int T, int K, int N, int epilogue) {
+GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim) {
   GemvPlan p;
   const int nacc = epilogue == kGemvSwiglu ? 2 : 1;
   static const int wg_env = getenv("SHAINET_HIP_GEMV_WGS") ? atoi(getenv("SHAINET_HIP_GEMV_WGS")) : 0;
@@ -249,6 +318,7 @@ GemvPlan plan_gemv(int T, int K, int N, int epilogue) {
   // most 16 along K; a matrix too narrow for that with 256-column tiles gets 64-column ones
   const int target = (wg_env > 0 ? wg_env : 1024) / nacc;
   p.rows_per_instr = ((N + 255) / 256) * 16 < target ? 4 : 1;
+  if (epilogue == kGemvQkvPrep && head_dim > 64) p.rows_per_instr = 1;  // a 64-column tile cannot hold a head
   const int cw = 256 / p.rows_per_instr;
   const int col_tiles = (N + cw - 1) / cw;
   int splits = (target + col_tiles - 1) / col_tiles;
@@ -272,13 +342,23 @@ GemvPlan plan_gemv(int T, int K, int N, int epilogue) {
 
 hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stream) {
   GemvArgs a = args;
-  if (a.T < 1 || a.T > 16 || a.K < 1 || a.N < 4 || (a.N & 3) || !a.x || !a.w || !a.y || a.x_stride < a.K)
+  if (a.T < 1 || a.T > 16 || a.K < 1 || a.N < 4 || (a.N & 3) || !a.x || !a.w || a.x_stride < a.K)
     return hipErrorInvalidValue;
+  if (!a.y && a.epilogue != kGemvQkvPrep) return hipErrorInvalidValue;
   if (p.rows_per_instr != 1 && p.rows_per_instr != 4) return hipErrorInvalidValue;
   if (p.rows_per_wave < 8 * p.rows_per_instr || p.rows_per_wave % (8 * p.rows_per_instr)) return hipErrorInvalidValue;
   if (p.splits > 1 && (!a.partials || !a.counters)) return hipErrorInvalidValue;
   if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
   if (a.epilogue != kGemvResidual) a.res = nullptr;
+  const bool prep = a.epilogue == kGemvQkvPrep;
+  if (prep) {
+    const GemvPrep &q = a.prep;
+    const int cw = 256 / p.rows_per_instr;
+    if (q.hd < 2 || q.hd > 128 || (q.hd & (q.hd - 1)) || cw % q.hd || q.H < 1 || q.KV < 1 ||
+        a.N != (q.H + 2 * q.KV) * q.hd || !q.rope_tab || !q.q_rot || !q.kc || !q.vc || q.start_pos < 0 ||
+        q.start_pos + a.T > q.cap)
+      return hipErrorInvalidValue;
+  }
   a.rows_per_wave = p.rows_per_wave;
   dim3 grid((unsigned)p.col_tiles, (unsigned)p.splits);
   const int nacc = a.epilogue == kGemvSwiglu ? 2 : 1;
@@ -286,25 +366,29 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
   const size_t stage = (size_t)tt * 4 * p.rows_per_wave * sizeof(float);
   const size_t red = (size_t)(3 * tt > 4 * nacc ? 3 * tt : 4 * nacc) * 64 * sizeof(f32x4);
   const size_t smem = stage > red ? stage : red;
-#define SHAINET_LAUNCH_GEMV(TT_, NACC_, RPI_) \
-  hipLaunchKernelGGL((gemv_fused_kernel<TT_, NACC_, RPI_>), grid, dim3(256), smem, stream, a)
-#define SHAINET_LAUNCH_GEMV_T(NACC_, RPI_)   \
-  do {                                       \
-    if (tt == 1)                             \
-      SHAINET_LAUNCH_GEMV(1, NACC_, RPI_);   \
-    else if (tt == 4)                        \
-      SHAINET_LAUNCH_GEMV(4, NACC_, RPI_);   \
-    else                                     \
-      SHAINET_LAUNCH_GEMV(16, NACC_, RPI_);  \
+#define SHAINET_LAUNCH_GEMV(TT_, NACC_, RPI_, PREP_) \
+  hipLaunchKernelGGL((gemv_fused_kernel<TT_, NACC_, RPI_, PREP_>), grid, dim3(256), smem, stream, a)
+#define SHAINET_LAUNCH_GEMV_T(NACC_, RPI_, PREP_)   \
+  do {                                              \
+    if (tt == 1)                                    \
+      SHAINET_LAUNCH_GEMV(1, NACC_, RPI_, PREP_);   \
+    else if (tt == 4)                               \
+      SHAINET_LAUNCH_GEMV(4, NACC_, RPI_, PREP_);   \
+    else                                            \
+      SHAINET_LAUNCH_GEMV(16, NACC_, RPI_, PREP_);  \
   } while (0)
-  if (nacc == 1 && p.rows_per_instr == 1)
-    SHAINET_LAUNCH_GEMV_T(1, 1);
+  if (prep && p.rows_per_instr == 1)
+    SHAINET_LAUNCH_GEMV_T(1, 1, true);
+  else if (prep)
+    SHAINET_LAUNCH_GEMV_T(1, 4, true);
+  else if (nacc == 1 && p.rows_per_instr == 1)
+    SHAINET_LAUNCH_GEMV_T(1, 1, false);
   else if (nacc == 1)
-    SHAINET_LAUNCH_GEMV_T(1, 4);
+    SHAINET_LAUNCH_GEMV_T(1, 4, false);
   else if (p.rows_per_instr == 1)
-    SHAINET_LAUNCH_GEMV_T(2, 1);
+    SHAINET_LAUNCH_GEMV_T(2, 1, false);
   else
-    SHAINET_LAUNCH_GEMV_T(2, 4);
+    SHAINET_LAUNCH_GEMV_T(2, 4, false);
 #undef SHAINET_LAUNCH_GEMV_T
 #undef SHAINET_LAUNCH_GEMV
   return hipGetLastError();

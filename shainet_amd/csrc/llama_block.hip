@@ -118,10 +118,24 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
   // q_full, k_new, v_new (llama_block.cr:253-255) as the three column blocks of one product
-  if ((rc = l->proj.project(x, l->d_model, l->w_qkv, l->qkv.p, T, l->d_model, wide, stream, pre))) return rc;
-  rc = shainet_attn_forward_strided(l->ctx, cache, nullptr, &T, 1, l->qkv.p, l->qkv.p + l->q_dim,
-                                    l->qkv.p + l->q_dim + l->kv_dim, wide, wide, wide, l->attn.p,
-                                    SHAINET_HIP_MEM_DEVICE);  // 256-296
+  const int hd = l->head_dim;
+  static const bool fuse_off = getenv("SHAINET_HIP_NO_FUSED_PREP") != nullptr;
+  if (!fuse_off && T <= 16 && (wide & 3) == 0 && hd >= 2 && hd <= 128 && (hd & (hd - 1)) == 0) {
+    // few rows: bias, QK-norm, RoPE and the cache append (256-286, 332-344) happen where the
+    // product's head rows are summed up; the attention kernel follows directly
+    GemvPrep where;
+    if ((rc = shainet_attn_begin_prepared(l->ctx, cache, T, &where))) return rc;
+    Fused qkv = pre;
+    qkv.epilogue = kGemvQkvPrep;
+    qkv.prep = &where;
+    if ((rc = l->proj.project(x, l->d_model, l->w_qkv, nullptr, T, l->d_model, wide, stream, qkv))) return rc;
+    rc = shainet_attn_finish_prepared(l->ctx, cache, T, l->attn.p);  // 287-296
+  } else {
+    if ((rc = l->proj.project(x, l->d_model, l->w_qkv, l->qkv.p, T, l->d_model, wide, stream, pre))) return rc;
+    rc = shainet_attn_forward_strided(l->ctx, cache, nullptr, &T, 1, l->qkv.p, l->qkv.p + l->q_dim,
+                                      l->qkv.p + l->q_dim + l->kv_dim, wide, wide, wide, l->attn.p,
+                                      SHAINET_HIP_MEM_DEVICE);  // 256-296
+  }
   if (rc) return rc;
   if (no_cache) {
     if ((rc = shainet_kv_cache_clear(cache, -1))) return rc;

@@ -12,6 +12,17 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
                                  const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                                  long long q_stride, long long k_stride, long long v_stride, float *out, int mem);
 
+// capi.hip: the two halves of shainet_attn_forward for one sequence (slot 0 of the
+// cache) when the kernel that produces q | k | v also does the bias / QK-norm / RoPE /
+// append step (the kGemvQkvPrep epilogue).  begin checks the capacity and says where
+// the prepared rows go; finish runs the attention kernel over them and counts the rows
+// into the cache.  Both are asynchronous on the context's stream.
+namespace shainet {
+struct GemvPrep;
+}
+int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, shainet::GemvPrep *where);
+int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out);
+
 // Device weight buffers of a block / a model, allocated on first request, for a loader
 // that fills them on the device (llama_block.hip, llama_model.hip).
 struct LlamaBlockBuffers {
@@ -40,6 +51,7 @@ struct Fused {
   bool norm = false;           // RMSNorm the rows of x first
   const float *gamma = nullptr;
   double eps = 0.0;
+  const GemvPrep *prep = nullptr;  // kGemvQkvPrep: where the head rows go (y may be null); at most 16 rows
 };
 
 // y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows

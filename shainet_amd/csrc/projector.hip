@@ -6,7 +6,8 @@
 
 #include <cstdlib>
 #include <cstring>
-#include <unordered_map>
+#include <array>
+#include <map>
 #include <vector>
 
 #include "../../include/shainet_hip_attn.h"
@@ -125,7 +126,7 @@ struct LtState {
   hipblasLtMatmulPreference_t pref = nullptr;
   void *workspace = nullptr;
   size_t workspace_cap = 0;
-  std::unordered_map<unsigned long long, LtShape> shapes;
+  std::map<std::array<long long, 4>, LtShape> shapes;  // (T, K, N, stride of x)
   void drop_shapes() {
     for (auto &kv : shapes) {
       if (kv.second.a) g_lt.layout_destroy(kv.second.a);
@@ -185,9 +186,7 @@ int Projector::gemm_lt(const float *x, long long x_stride, const float *w, float
     }
   }
   if (lt_broken) return 0;
-  // the stride of x is part of the key; T, K, N below 2^20 and strides below 2^24 keep the fields apart
-  const unsigned long long key = ((unsigned long long)T << 44) ^ ((unsigned long long)K << 24) ^
-                                 ((unsigned long long)N << 4) ^ ((unsigned long long)x_stride << 40);
+  const std::array<long long, 4> key = {T, K, N, x_stride};
   if (lt->shapes.size() > 512) lt->drop_shapes();
   auto it = lt->shapes.find(key);
   if (it == lt->shapes.end()) {
@@ -256,6 +255,8 @@ int Projector::gemm(const float *x, long long x_stride, const float *w, float *y
 int Projector::project(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N,
                        hipStream_t stream, const Fused &f) {
   const bool swiglu = f.epilogue == kGemvSwiglu;
+  if (f.epilogue == kGemvQkvPrep && (!f.prep || T > 16 || (N & 3)))
+    return llama_fail(SHAINET_HIP_ERR_ARGUMENT, "the fused q | k | v epilogue takes at most 16 rows");
   if (T <= 16 && (N & 3) == 0) {
     const float *xin = x;
     long long xs = x_stride;
@@ -268,7 +269,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
       xs = K;
       norm = false;
     }
-    const GemvPlan p = plan_gemv(T, K, N, f.epilogue);
+    const GemvPlan p = plan_gemv(T, K, N, f.epilogue, f.prep ? f.prep->hd : 0);
     if (!scratch.reserve(p.partial_floats)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
     if ((size_t)p.col_tiles > counters_cap) {
       size_t want = counters_cap ? counters_cap : 1024;
@@ -298,6 +299,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.K = K;
     a.N = N;
     a.epilogue = f.epilogue;
+    if (f.prep) a.prep = *f.prep;
     hipError_t e = launch_gemv(a, p, stream);
     if (e != hipSuccess)
       return llama_fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemv launch: ") + hipGetErrorString(e));

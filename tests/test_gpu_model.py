@@ -87,6 +87,65 @@ def test_block_every_small_row_count(hip):
     assert blk.cache_len == ob.cache_len == 68
 
 
+def test_first_rows_of_a_new_cache_survive_its_zero_fill(hip):
+    # a new cache is zero-filled; the fill must be over before the first rows are appended (a fill
+    # that ran late wiped row 0 now and then): many fresh blocks, same input, same bits every time
+    first = None
+    for _ in range(30):
+        blk, _, _, r, _ = _block_pair(hip, 128, 8, 2, 64, 344, 1e4, seed=128, norm=True, bias=True)
+        y = blk.forward(r.standard_normal((1, 128)).astype(np.float32))   # creates the scratch cache
+        z = blk.forward_cached(r.standard_normal((1, 128)).astype(np.float32))
+        blk.close()
+        got = np.concatenate([y, z]).view(np.uint32)
+        if first is None:
+            first = got
+        assert np.array_equal(got, first)
+
+
+_FUSED_PREP_CHILD = """
+import sys
+import numpy as np
+sys.path.insert(0, {root!r})
+sys.path.insert(0, {tests!r})
+import shainet_amd as sa
+import test_gpu_model as t
+outs = t._fused_prep_sequence(sa, {hd})
+np.savez({out!r}, *outs)
+"""
+
+
+def _fused_prep_sequence(hip, hd):
+    # the oracle half of the pair is not used here
+    blk, _, _, r, _ = _block_pair(hip, 256, 4, 2, hd, 512, 1e4, seed=23 + hd, norm=True, bias=True)
+    outs = []
+    for T in (5, 1, 1, 16, 3, 1, 40, 1):
+        outs.append(blk.forward_cached(r.standard_normal((T, 256)).astype(np.float32)))
+    return outs
+
+
+@pytest.mark.parametrize("hd", [128, 64, 32])
+def test_qkv_product_with_prep_inside_equals_separate_prep_bit_for_bit(hip, hd, tmp_path):
+    # up to 16 rows the q | k | v product applies bias, QK-norm, RoPE and the cache append itself;
+    # a process with that switched off runs the separate prep kernel on the same product: every
+    # later output depends on the cache contents, so equal bits mean equal caches.  (head_dim 128
+    # makes the fused product use 256-column tiles where the plain one takes 64-column tiles: the
+    # sums are added in another order there and only the tolerance holds.)
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    out = str(tmp_path / "unfused.npz")
+    code = _FUSED_PREP_CHILD.format(root=os.path.dirname(here), tests=here, hd=hd, out=out)
+    env = dict(os.environ, SHAINET_HIP_NO_FUSED_PREP="1")
+    subprocess.run([sys.executable, "-c", code], check=True, env=env, timeout=300)
+    unfused = np.load(out)
+    fused = _fused_prep_sequence(hip, hd)
+    for i, y in enumerate(fused):
+        if hd <= 64:
+            assert np.array_equal(y.view(np.uint32), unfused[f"arr_{i}"].view(np.uint32)), f"call {i}"
+        else:
+            rm.assert_close(y, unfused[f"arr_{i}"], ATOL, RTOL, f"call {i}")
+
+
 def test_block_many_rows_both_library_gemms(hip):
     # more than 16 rows: rocBLAS below 256 rows of a small weight matrix, hipBLASLt from 256 rows on
     blk, ob, p, r, eps = _block_pair(hip, 128, 8, 2, 64, 344, 1e4, seed=5, norm=True, bias=True)
