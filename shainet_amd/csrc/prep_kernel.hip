@@ -13,6 +13,8 @@
 #include "attn_kernels.hpp"
 #include "prep_math.hpp"
 
+#include <stdint.h>
+
 #pragma clang fp contract(off)
 
 namespace shainet {
@@ -111,6 +113,48 @@ __global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st,
   }
 }
 
+// Many rows without QK-norm (prefill of the Llama shapes): nothing crosses lanes, so a
+// lane takes four neighbouring pairs of one head row with 16-byte accesses.  head_dim is
+// a multiple of 8 and every row start is 16-byte aligned.  Same products and sums as
+// norm_rotate_pair without weights.
+__global__ __launch_bounds__(256) void prep_rows_vec_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens,
+                                                            long long n_items) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_items) return;
+  const int half = sh.hd >> 1, tpr = half >> 2, rows = sh.H + 2 * sh.KV;
+  const int j = (int)(idx % tpr);
+  const long long row_g = idx / tpr;
+  const int token = (int)(row_g / rows), r = (int)(row_g - (long long)token * rows);
+  const RowRef rr = locate_row(a, st, sh, token, r, total_tokens);
+  const int i0 = 4 * j;
+  float4 x0 = *(const float4 *)(rr.src + i0), x1 = *(const float4 *)(rr.src + half + i0);
+  if (rr.bias) {
+    const float4 b0 = *(const float4 *)(rr.bias + i0), b1 = *(const float4 *)(rr.bias + half + i0);
+    x0 = float4{x0.x + b0.x, x0.y + b0.y, x0.z + b0.z, x0.w + b0.w};
+    x1 = float4{x1.x + b1.x, x1.y + b1.y, x1.z + b1.z, x1.w + b1.w};
+  }
+  if (rr.rotate) {
+    const float4 *cs = (const float4 *)(a.rope_tab + (long long)rr.pos * half + i0);
+    const float4 cs01 = cs[0], cs23 = cs[1];  // (cos, sin) of pairs i0, i0 + 1 and i0 + 2, i0 + 3
+    float4 y0, y1;
+#define SHAINET_ROTATE(f, c, s)            \
+  {                                        \
+    const float p0 = x0.f * c, p1 = x1.f * s, p2 = x1.f * c, p3 = x0.f * s; \
+    y0.f = p0 - p1;                        \
+    y1.f = p2 + p3;                        \
+  }
+    SHAINET_ROTATE(x, cs01.x, cs01.y)
+    SHAINET_ROTATE(y, cs01.z, cs01.w)
+    SHAINET_ROTATE(z, cs23.x, cs23.y)
+    SHAINET_ROTATE(w, cs23.z, cs23.w)
+#undef SHAINET_ROTATE
+    x0 = y0;
+    x1 = y1;
+  }
+  *(float4 *)(rr.dst + i0) = x0;
+  *(float4 *)(rr.dst + half + i0) = x1;
+}
+
 // Any head_dim (odd ones included): one wavefront per head row.
 __global__ __launch_bounds__(256) void prep_rows_generic_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
   const int lane = threadIdx.x & 63;
@@ -188,6 +232,20 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
   // (prefill): four rows per wavefront amortise the load latency
   const int rows_per_wave = fast && (long long)total_tokens * rows >= 8192 ? 4 : 1;
   const int per_wg = 4 * rows_per_wave;
+  const auto aligned16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = !a.q_norm && !a.k_norm && (sh.hd & 7) == 0 && (long long)total_tokens * rows >= 8192 &&
+                   ((a.q_stride | a.k_stride | a.v_stride) & 3) == 0 && aligned16(a.q) && aligned16(a.k) &&
+                   aligned16(a.v) && aligned16(a.q_rot) && aligned16(a.kc) && aligned16(a.vc) && aligned16(a.b_q) &&
+                   aligned16(a.b_k) && aligned16(a.b_v) && aligned16(a.rope_tab);
+  if (vec) {
+    const long long n_items = (long long)total_tokens * rows * (sh.hd >> 3);
+    const long long blocks = (n_items + 255) / 256;
+    if (blocks <= 0x7fffffffLL) {
+      hipLaunchKernelGGL(prep_rows_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, st, sh,
+                         total_tokens, n_items);
+      return hipGetLastError();
+    }
+  }
   // blockIdx.y is the token; a launch takes at most 65535 of them
   for (int t0 = 0; t0 < total_tokens; t0 += 65535) {
     const int nt = total_tokens - t0 < 65535 ? total_tokens - t0 : 65535;

@@ -154,6 +154,26 @@ def test_rotated_q_and_cache_are_bit_identical(hip, H, KV, hd, theta, norm, bias
     assert k0.shape == (15, hd) and not np.array_equal(k0[1], k0[2])
 
 
+@pytest.mark.parametrize("H,KV,hd,bias", [(32, 8, 64, True), (8, 2, 128, False), (8, 4, 8, True), (4, 1, 256, True)])
+def test_many_rows_without_norm_take_wide_accesses_same_bits(hip, H, KV, hd, bias):
+    # from 8192 head rows on, rows without QK-norm go through a kernel with 16-byte accesses:
+    # ragged batch, bias, start positions above zero; rotated Q and both caches bit for bit
+    per_token = H + 2 * KV
+    T0 = 8192 // per_token + 3
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, False, bias, batch=3, capacity=T0 + 64, seed=hd)
+    for new in ([T0 // 2 + 3, 5, T0 // 2 + 1], [1, T0, 7]):
+        parts = [rows(r, T, H, KV, hd) for T in new]
+        q, k, v = (np.concatenate([p[i] for p in parts]) for i in range(3))
+        ctx.forward(cache, q, k, v, new)
+        want_q = []
+        for s, pt in enumerate(parts):
+            blocks[s].attention_cached_qkv(*pt, keep_q_rot=True, threads=16)
+            want_q.append(blocks[s].last_q_rot)
+        got_q = ctx.last_q_rot(sum(new))
+        assert np.array_equal(got_q.view(np.uint32), np.concatenate(want_q).view(np.uint32)), "rotated Q bits differ"
+    check_cache_bits(cache, blocks)
+
+
 # ------------------------------------------------------------------ decode (split-K kernel)
 def test_config1_llama1b_decode_on_prefilled_cache(hip):
     # Llama-3.2-1B head geometry, cache pre-filled to 512 positions, one new row
