@@ -257,8 +257,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     }
     // Every wavefront is done with the O rows parked in LDS (the next segment's K
     // tiles land there).  Partials are written through to device-coherent memory
-    // (coherent_store); the barrier also waits for this workgroup's stores to be
-    // acknowledged before its arrival is counted.
+    // (coherent_store); each wavefront waits for its stores to be acknowledged
+    // (s_waitcnt vmcnt(0): the barrier alone does not) before the arrival is counted.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     if (!whole_pair) {
       // The last workgroup to deliver a partial of this pair merges them all.  The

@@ -239,7 +239,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   }
 
   // ---- the last workgroup of this column tile adds the partials in a fixed order
-  __syncthreads();  // the partial stores above are acknowledged before the arrival is counted
+  // the partial stores above are acknowledged (s_waitcnt vmcnt(0): the barrier alone does
+  // not wait for them) before the arrival is counted
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
   if (threadIdx.x == 0) {
     const int old = atomicAdd(&a.counters[blockIdx.x], 1);
     last_flag = old == splits - 1;
