@@ -395,6 +395,8 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
 }
 
 // Merge the key chunks of one (row block, kv head): online-softmax combine per row.
+// Four workgroups per block (32 of its 128 virtual rows each, blockIdx.y) and up to eight
+// chunks' loads in flight per thread: the kernel is bound by load latency, not by bytes.
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ part_o,
                                                               const float *__restrict__ part_ml,
                                                               float *__restrict__ out, SeqTable st, Shape sh,
@@ -405,20 +407,38 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__res
   const int g = sh.g, hd = sh.hd, hd4 = hd >> 2;
   const int VR = st.n_new[s] * g;
   const long long base = ((long long)item * sh.KV + kvh) * ns * 128;
-  for (int idx = threadIdx.x; idx < 128 * hd4; idx += 256) {
-    const int vl = idx / hd4, d4 = idx - vl * hd4;
+  for (int idx = threadIdx.x; idx < 32 * hd4; idx += 256) {
+    const int vl = blockIdx.y * 32 + idx / hd4, d4 = idx % hd4;
     const int v = vb * 128 + vl;
     if (v >= VR) continue;
     const int row = v / g, hg = v - row * g;
     float mm = -INFINITY;
-    for (int k = 0; k < ns; ++k) mm = fmaxf(mm, part_ml[2 * (base + (long long)k * 128 + vl)]);
+    for (int k0 = 0; k0 < ns; k0 += 8) {
+      float mk[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) mk[u] = part_ml[2 * (base + (long long)min(k0 + u, ns - 1) * 128 + vl)];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) mm = fmaxf(mm, mk[u]);
+    }
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float ls = 0.f;
-    for (int k = 0; k < ns; ++k) {
-      const long long pi = base + (long long)k * 128 + vl;
-      const float f = fast_exp2((part_ml[2 * pi] - mm) * c);  // 0 for a chunk that saw no visible key
-      acc += f * *(const f32x4 *)(part_o + pi * hd + 4 * d4);
-      ls += f * part_ml[2 * pi + 1];
+    for (int k0 = 0; k0 < ns; k0 += 8) {
+      f32x4 x[8];
+      float mk[8], lk[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const long long pi = base + (long long)min(k0 + u, ns - 1) * 128 + vl;
+        x[u] = *(const f32x4 *)(part_o + pi * hd + 4 * d4);
+        mk[u] = part_ml[2 * pi];
+        lk[u] = part_ml[2 * pi + 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        // 0 for a chunk that saw no visible key, and for the clamped repeats past the last chunk
+        const float f = k0 + u < ns ? fast_exp2((mk[u] - mm) * c) : 0.f;
+        acc += f * x[u];
+        ls += f * lk[u];
+      }
     }
     *(f32x4 *)(out + ((long long)(st.tok_off[s] + row) * sh.H + kvh * g + hg) * hd + 4 * d4) = acc * (1.0f / ls);
   }
@@ -600,7 +620,7 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
 #undef SHAINET_LAUNCH_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || ns == 1) return e;
-  hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV)), dim3(256), 0, stream, part_o, part_ml,
+  hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, part_o, part_ml,
                      out, st, sh, ns, c);
   return hipGetLastError();
 }

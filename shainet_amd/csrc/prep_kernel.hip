@@ -155,6 +155,92 @@ __global__ __launch_bounds__(256) void prep_rows_vec_kernel(PrepArgs a, SeqTable
   *(float4 *)(rr.dst + half + i0) = x1;
 }
 
+// Many rows with QK-norm (prefill of the Qwen3 shapes).  The sum of squares of a head row
+// must be added up in the reference's order, one fp32 add per element, which leaves a
+// wavefront per row waiting on a chain of hd dependent adds (25 us for 20 480 rows of 128).
+// Here a workgroup takes ROWS head rows through LDS: all threads load them (bias added),
+// then one lane per row walks its row (row stride hd + 1 floats: no bank conflicts), then
+// all threads normalise, rotate and store pair by pair with coalesced accesses.  The same
+// products and sums as norm_rotate_pair, the same bits.
+template <int ROWS>
+__global__ __launch_bounds__(256) void prep_rows_norm_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens,
+                                                             long long n_rows) {
+  extern __shared__ float xs[];  // [ROWS][hd + 1]
+  __shared__ const float *src_s[ROWS], *bias_s[ROWS], *w_s[ROWS];
+  __shared__ float *dst_s[ROWS];
+  __shared__ int pos_s[ROWS];
+  __shared__ bool rot_s[ROWS];
+  __shared__ float inv_s[ROWS];
+  const int hd = sh.hd, half = hd >> 1, stride = hd + 1, per_token = sh.H + 2 * sh.KV;
+  const long long row0 = (long long)blockIdx.x * ROWS;
+  const int t = threadIdx.x;
+  if (t < ROWS) {
+    const long long row_g = row0 + t;
+    RowRef rr;
+    rr.src = nullptr;
+    if (row_g < n_rows) {
+      const int token = (int)(row_g / per_token);
+      rr = locate_row(a, st, sh, token, (int)(row_g - (long long)token * per_token), total_tokens);
+    }
+    src_s[t] = rr.src;
+    if (rr.src) {
+      bias_s[t] = rr.bias;
+      w_s[t] = rr.w;
+      dst_s[t] = rr.dst;
+      pos_s[t] = rr.pos;
+      rot_s[t] = rr.rotate;
+    }
+  }
+  __syncthreads();
+  for (int idx = t; idx < ROWS * hd; idx += 256) {
+    const int r = idx / hd, d = idx - r * hd;
+    const float *src = src_s[r];
+    float x = 0.0f;
+    if (src) {
+      x = src[d];
+      const float *bias = bias_s[r];
+      if (bias) x = x + bias[d];
+    }
+    xs[r * stride + d] = x;
+  }
+  __syncthreads();
+  if (t < ROWS && src_s[t] && w_s[t]) {  // llama_block.cr:626-633
+    const float *row = xs + t * stride;
+    float ss = 0.0f;
+#pragma unroll 8
+    for (int d = 0; d < hd; ++d) {
+      const float v = row[d];
+      const float sq = v * v;
+      ss = ss + sq;
+    }
+    const float mean = ss / (float)hd;
+    inv_s[t] = (float)(1.0 / sqrt((double)mean + a.eps));
+  }
+  __syncthreads();
+  for (int idx = t; idx < ROWS * half; idx += 256) {
+    const int r = idx / half, i = idx - r * half;
+    if (!src_s[r]) continue;
+    float x0 = xs[r * stride + i], x1 = xs[r * stride + i + half];
+    float *dst = dst_s[r];
+    if (rot_s[r]) {
+      const float *w = w_s[r];
+      if (w) {  // 636
+        const float inv = inv_s[r];
+        x0 = x0 * inv;
+        x0 = x0 * w[i];
+        x1 = x1 * inv;
+        x1 = x1 * w[i + half];
+      }
+      const float2 cs = a.rope_tab[(long long)pos_s[r] * half + i];
+      const float p0 = x0 * cs.x, p1 = x1 * cs.y, p2 = x1 * cs.x, p3 = x0 * cs.y;
+      x0 = p0 - p1;
+      x1 = p2 + p3;
+    }
+    dst[i] = x0;
+    dst[i + half] = x1;
+  }
+}
+
 // Any head_dim (odd ones included): one wavefront per head row.
 __global__ __launch_bounds__(256) void prep_rows_generic_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
   const int lane = threadIdx.x & 63;
@@ -237,6 +323,17 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
                    ((a.q_stride | a.k_stride | a.v_stride) & 3) == 0 && aligned16(a.q) && aligned16(a.k) &&
                    aligned16(a.v) && aligned16(a.q_rot) && aligned16(a.kc) && aligned16(a.vc) && aligned16(a.b_q) &&
                    aligned16(a.b_k) && aligned16(a.b_v) && aligned16(a.rope_tab);
+  if (fast && (a.q_norm || a.k_norm) && (long long)total_tokens * rows >= 8192) {
+    constexpr int kRows = 16;  // small groups: many workgroups per compute unit hide each other's latencies
+    const long long n_rows = (long long)total_tokens * rows;
+    const long long blocks = (n_rows + kRows - 1) / kRows;
+    if (blocks <= 0x7fffffffLL) {
+      const size_t lds = (size_t)kRows * (sh.hd + 1) * sizeof(float);
+      hipLaunchKernelGGL(prep_rows_norm_kernel<kRows>, dim3((unsigned)blocks), dim3(256), lds, stream, a, st, sh,
+                         total_tokens, n_rows);
+      return hipGetLastError();
+    }
+  }
   if (vec) {
     const long long n_items = (long long)total_tokens * rows * (sh.hd >> 3);
     const long long blocks = (n_items + 255) / 256;

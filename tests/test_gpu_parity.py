@@ -154,13 +154,17 @@ def test_rotated_q_and_cache_are_bit_identical(hip, H, KV, hd, theta, norm, bias
     assert k0.shape == (15, hd) and not np.array_equal(k0[1], k0[2])
 
 
-@pytest.mark.parametrize("H,KV,hd,bias", [(32, 8, 64, True), (8, 2, 128, False), (8, 4, 8, True), (4, 1, 256, True)])
-def test_many_rows_without_norm_take_wide_accesses_same_bits(hip, H, KV, hd, bias):
-    # from 8192 head rows on, rows without QK-norm go through a kernel with 16-byte accesses:
-    # ragged batch, bias, start positions above zero; rotated Q and both caches bit for bit
+@pytest.mark.parametrize("H,KV,hd,norm,bias", [
+    (32, 8, 64, False, True), (8, 2, 128, False, False), (8, 4, 8, False, True), (4, 1, 256, False, True),
+    (32, 8, 128, True, False), (8, 2, 64, True, True), (8, 4, 16, True, True), (6, 3, 30, True, False),
+])
+def test_many_rows_take_the_bulk_prep_kernels_same_bits(hip, H, KV, hd, norm, bias):
+    # from 8192 head rows on: without QK-norm a kernel with 16-byte accesses, with QK-norm one that
+    # walks each row's sum of squares in LDS.  Ragged batch, bias, start positions above zero;
+    # rotated Q and both caches bit for bit
     per_token = H + 2 * KV
     T0 = 8192 // per_token + 3
-    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, False, bias, batch=3, capacity=T0 + 64, seed=hd)
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, norm, bias, batch=3, capacity=T0 + 64, seed=hd)
     for new in ([T0 // 2 + 3, 5, T0 // 2 + 1], [1, T0, 7]):
         parts = [rows(r, T, H, KV, hd) for T in new]
         q, k, v = (np.concatenate([p[i] for p in parts]) for i in range(3))
