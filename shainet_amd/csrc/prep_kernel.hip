@@ -323,6 +323,7 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
                    ((a.q_stride | a.k_stride | a.v_stride) & 3) == 0 && aligned16(a.q) && aligned16(a.k) &&
                    aligned16(a.v) && aligned16(a.q_rot) && aligned16(a.kc) && aligned16(a.vc) && aligned16(a.b_q) &&
                    aligned16(a.b_k) && aligned16(a.b_v) && aligned16(a.rope_tab);
+  // (for a decode step's few hundred rows the one-wavefront-per-row kernel is the shorter one: 5.8 against 10 us)
   if (fast && (a.q_norm || a.k_norm) && (long long)total_tokens * rows >= 8192) {
     constexpr int kRows = 16;  // small groups: many workgroups per compute unit hide each other's latencies
     const long long n_rows = (long long)total_tokens * rows;
