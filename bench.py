@@ -101,7 +101,8 @@ class Workload:
         ctx.profile(True)
         for i in range(steps):
             step(warmup + steps + i)
-        k_ms, launches = ctx.profile_read()
+        samples = ctx.profile_samples(steps + 8)
+        k_ms, launches = float(samples.sum()), len(samples)
         ctx.profile(False)
         vis_wall = [[L + warmup + i + 1 for L in self.lens] for i in range(steps)]
         vis_prof = [[L + warmup + steps + i + 1 for L in self.lens] for i in range(steps)]
@@ -109,7 +110,11 @@ class Workload:
         b_prof = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_prof) / steps
         us = wall / steps * 1e6
         kus = k_ms / max(launches, 1) * 1e3
-        return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "launches": launches,
+        import numpy as np
+
+        pct = [float(x) * 1e3 for x in np.percentile(samples, (10, 50, 90))] if launches else [0.0] * 3
+        return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "kernel_us_p10": pct[0],
+                "kernel_us_p50": pct[1], "kernel_us_p90": pct[2], "launches": launches,
                 "bytes_per_step": b_wall, "step_gbps": b_wall / us / 1e3, "kernel_gbps": b_prof / kus / 1e3,
                 "kernel_bytes": b_prof}
 
@@ -393,7 +398,10 @@ def main():
         "hbm_gbps": round(h["step_gbps"], 1),
         "roofline": {"bound": "hbm", "kernel": "decode_splitk_kernel<128, 4>", "achieved": round(h["kernel_gbps"], 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(h["kernel_gbps"] / HBM_PEAK_GBPS, 4),
-                     "kernel_us": round(h["kernel_us"], 2), "bytes_per_launch": int(h["kernel_bytes"]),
+                     "kernel_us": round(h["kernel_us"], 2), "kernel_us_p10_p50_p90": [round(h["kernel_us_p10"], 2),
+                                                                                      round(h["kernel_us_p50"], 2),
+                                                                                      round(h["kernel_us_p90"], 2)],
+                     "bytes_per_launch": int(h["kernel_bytes"]),
                      "traffic": load_traffic("decode_splitk_kernel<128, 4>", head.name, h["kernel_bytes"])},
         "cpu_baseline": cpu,
         "workloads": {k_: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in r.items()

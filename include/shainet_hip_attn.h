@@ -317,9 +317,12 @@ int shainet_hf_load_llama(const char *model_dir, shainet_llama_model **out);
  * kernel or the generic kernel; not the prep or combine kernels) with HIP events
  * on the context's stream.  shainet_attn_profile_read waits for the stream,
  * returns the summed kernel time in milliseconds and the number of launches
- * since the last read, and resets both.  No counterpart in the reference. */
+ * since the last read, and resets both; shainet_attn_profile_samples does the same
+ * but hands back the time of each launch (the first `capacity` of them; *launches
+ * is the number there were).  No counterpart in the reference. */
 int shainet_attn_profile(shainet_attn_ctx *ctx, int enable);
 int shainet_attn_profile_read(shainet_attn_ctx *ctx, double *total_ms, int *launches);
+int shainet_attn_profile_samples(shainet_attn_ctx *ctx, float *ms_out, int capacity, int *launches);
 
 /* Plain streaming kernels of known size (device pointers, n floats, n % 4 == 0,
  * grid-stride over `workgroups` workgroups of 256 lanes, on `stream`): a copy

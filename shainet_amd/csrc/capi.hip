@@ -677,15 +677,14 @@ int shainet_attn_profile(shainet_attn_ctx *c, int enable) {
   return SHAINET_HIP_OK;
 }
 
-int shainet_attn_profile_read(shainet_attn_ctx *c, double *total_ms, int *launches) {
-  if (!c || !total_ms || !launches) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+int shainet_attn_profile_samples(shainet_attn_ctx *c, float *ms_out, int capacity, int *launches) {
+  if (!c || !launches || capacity < 0 || (capacity > 0 && !ms_out)) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   HIP_TRY(hipStreamSynchronize(c->stream));
-  double sum = 0.0;
   int n = 0;
   for (size_t i = 0; i + 1 < c->prof_events.size(); i += 2) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, c->prof_events[i], c->prof_events[i + 1]) == hipSuccess) {
-      sum += ms;
+      if (n < capacity) ms_out[n] = ms;
       ++n;
     }
     (void)hipEventDestroy(c->prof_events[i]);
@@ -693,6 +692,18 @@ int shainet_attn_profile_read(shainet_attn_ctx *c, double *total_ms, int *launch
   }
   (void)hipGetLastError();
   c->prof_events.clear();
+  *launches = n;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_attn_profile_read(shainet_attn_ctx *c, double *total_ms, int *launches) {
+  if (!c || !total_ms || !launches) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  std::vector<float> ms(c->prof_events.size() / 2 + 1);
+  int n = 0;
+  const int rc = shainet_attn_profile_samples(c, ms.data(), (int)ms.size(), &n);
+  if (rc) return rc;
+  double sum = 0.0;
+  for (int i = 0; i < n && i < (int)ms.size(); ++i) sum += ms[i];
   *total_ms = sum;
   *launches = n;
   return SHAINET_HIP_OK;

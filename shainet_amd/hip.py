@@ -128,6 +128,7 @@ _SIGNATURES = {
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
     "shainet_attn_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), _i32p]),
+    "shainet_attn_profile_samples": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, _i32p]),
 }
 
 
@@ -273,6 +274,15 @@ class AttnContext:
         ms, n = C.c_double(0), C.c_int(0)
         _check(lib().shainet_attn_profile_read(self._h, C.byref(ms), C.byref(n)))
         return ms.value, n.value
+
+    def profile_samples(self, capacity=4096):
+        """Attention-kernel milliseconds of each launch since the last read (numpy float32)."""
+        import numpy as np
+
+        out = np.zeros(capacity, np.float32)
+        n = C.c_int(0)
+        _check(lib().shainet_attn_profile_samples(self._h, out.ctypes.data, capacity, C.byref(n)))
+        return out[:min(n.value, capacity)]
 
     def inv_freq(self):
         import numpy as np
