@@ -3,6 +3,8 @@
 Bar (fp32): |gpu - oracle| <= 1e-4 + 1e-3*|oracle| elementwise; rotated Q rows and
 cache contents (RoPE positions, cache indexing) bit-identical.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -501,3 +503,14 @@ def test_layer_argument_errors(hip):
     blk.set_qk_norm(np.ones(7), np.ones(8))                 # llama_block.cr:618
     with pytest.raises(hip.ArgumentError):
         blk.attention_cached(np.zeros((1, 32), np.float32))
+
+
+def test_c_abi_from_plain_c(hip):
+    # tests/cabi_smoke.c, compiled by __graft_entry__.build(): the fused entry points called from C,
+    # checked against closed forms (one key: out == V; two keys: a two-way softmax in double)
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi_smoke")
+    assert os.path.exists(exe), "tests/cabi_smoke is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    done = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0 and "cabi_smoke ok" in done.stdout, done.stdout + done.stderr
