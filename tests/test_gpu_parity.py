@@ -510,7 +510,11 @@ def test_c_abi_from_plain_c(hip):
     # checked against closed forms (one key: out == V; two keys: a two-way softmax in double)
     import subprocess
 
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi_smoke")
-    assert os.path.exists(exe), "tests/cabi_smoke is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = os.path.join(here, "cabi_smoke")
+    if not os.path.exists(exe):  # normally built by __graft_entry__.build(); a fraction of a second with gcc
+        lib_dir = os.path.dirname(hip.library_path())
+        subprocess.run(["gcc", "-O1", "-Wall", "-o", exe, os.path.join(here, "cabi_smoke.c"), "-L" + lib_dir,
+                        "-lshainet_hip_kernels", "-lm", "-Wl,-rpath,$ORIGIN/../shainet_amd/lib"], check=True)
     done = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert done.returncode == 0 and "cabi_smoke ok" in done.stdout, done.stdout + done.stderr
