@@ -366,6 +366,8 @@ def main():
         ("llama1b_prefill_t2048", 32, 8, 64, 5e5, False, [0], 2048, small),
         ("llama1b_prefill_t8192", 32, 8, 64, 5e5, False, [0], 8192, max(5, K // 20)),
         ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512, max(5, K // 10)),
+        # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
+        ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048, max(5, K // 10)),
     ]
     for name, H, KV, hd, th, norm, lens, T, k_ in prefill_cfgs:
         if want(name):
