@@ -333,6 +333,31 @@ def test_batched_prefill_mixed_lengths(hip):
     check_cache_bits(cache, blocks)
 
 
+def test_maximum_batch_ragged_and_call_errors(hip):
+    # 64 sequences (the limit per call): fresh, short and longer ones in one call, a prefill call with
+    # mixed row counts (1 row included), then a decode call; then what a call must refuse
+    H, KV, hd, B = 8, 2, 64, 64
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, bias=True, batch=B, capacity=96, seed=64)
+    first = [int(x) for x in r.integers(1, 40, B)]
+    first[0], first[1], first[63] = 1, 39, 1
+    check_step(ctx, cache, blocks, r, first, threads=16, what="64 sequences, 1..39 rows each")
+    check_step(ctx, cache, blocks, r, [1] * B, threads=16, what="64 sequences, decode")
+    some = [5, 17, 40, 63, 0]
+    check_step(ctx, cache, blocks, r, [1, 3, 1, 2, 1], seq_ids=some, what="five of them, out of order")
+    check_cache_bits(cache, blocks)
+    q, k, v = rows(r, 2, H, KV, hd)
+    for bad_ids, bad_new in (([3, 3], [1, 1]), ([64, 0], [1, 1]), ([-1, 0], [1, 1]), ([0, 1], [1, 0])):
+        before = [cache.len(s) for s in range(B)]
+        n = sum(bad_new)
+        with pytest.raises(hip.ArgumentError):
+            ctx.forward(cache, q[:n], k[:n], v[:n], bad_new, bad_ids)
+        assert [cache.len(s) for s in range(B)] == before, "a refused call changed a length"
+    with pytest.raises(hip.HipError):  # capacity: nothing appended
+        qq, kk, vv = rows(r, 96, H, KV, hd)
+        ctx.forward(cache, qq, kk, vv, [96], [7])
+    assert cache.len(7) == blocks[7].cache_len
+
+
 # ------------------------------------------------------------------ properties at full size
 def test_full_size_properties_prefill_8192(hip):
     """T = 8192 (Llama-1B geometry): too slow for the scalar oracle on every row, so check
