@@ -358,6 +358,38 @@ def test_maximum_batch_ragged_and_call_errors(hip):
     assert cache.len(7) == blocks[7].cache_len
 
 
+def test_cache_slot_beyond_four_gib(hip):
+    # the last slot of a large cache starts 4.3 GB into each tensor: offsets must not be 32-bit
+    H, KV, hd, cap = 32, 8, 128, 131072
+    r = np.random.default_rng(5)
+    qn, kn = ((1 + 0.02 * r.standard_normal(hd)).astype(np.float32) for _ in range(2))
+    ctx = hip.AttnContext(H, KV, hd, rope_theta=1e6, q_norm=qn, k_norm=kn, eps=1e-6)
+    cache = hip.KVCache(ctx, 9, cap)
+    blk = orc.Block(H * hd, H, KV, hd, eps=1e-6, rope_theta=1e6)
+    blk.set_qk_norm(qn, kn)
+    for T in (300, 1, 1):  # prefill kernel, then the split-K decode kernel
+        q, k, v = rows(r, T, H, KV, hd)
+        got = ctx.forward(cache, q, k, v, [T], [8])
+        rm.assert_close(got, blk.attention_cached_qkv(q, k, v, threads=16), ATOL, RTOL, f"T={T} in slot 8")
+    for c in (0, KV - 1):
+        kd, vd = cache.read(8, c, 0, 302)
+        assert np.array_equal(kd, blk.k_cache(c)) and np.array_equal(vd, blk.v_cache(c))
+    assert cache.len(8) == 302 and cache.len(0) == 0
+    cache.close()
+    ctx.close()
+
+
+def test_decode_context_131072(hip):
+    # one sequence of 131 072 cached positions (65 536 tiles over the 8 kv heads), one new row
+    H, KV, hd, S = 32, 8, 128, 131072
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, capacity=S + 8, seed=13)
+    kf, vf = (r.standard_normal((KV, S, hd), dtype=np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    assert check_step(ctx, cache, blocks, r, [1], threads=16) < 1e-4
+    assert cache.len(0) == S + 1
+
+
 # ------------------------------------------------------------------ properties at full size
 def test_full_size_properties_prefill_8192(hip):
     """T = 8192 (Llama-1B geometry): too slow for the scalar oracle on every row, so check
