@@ -119,6 +119,21 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   const int ldw = NACC * N;  // row pitch of W
   const bool have_col = col < N;  // N is a multiple of 4
 
+  // The first eight row loads of W do not depend on x: they are issued before the prologue
+  // and land while the norm is computed and x is staged (a product of 128 rows per
+  // workgroup with 4 rows per instruction is these eight loads and nothing more).
+  const int kk0 = wave * rpw;  // this wavefront's rows, relative to k_wg
+  f32x4 r_first[NACC][8];
+  const bool have_first = have_col && k_wg + kk0 < K;
+  if (have_first) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int row = min(k_wg + kk0 + u * RPI + sub, K - 1);
+#pragma unroll
+      for (int c = 0; c < NACC; ++c) r_first[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+    }
+  }
+
   // ---- prologue: the x values of this workgroup's K range, normalised if asked;
   // zero beyond K and beyond T, so that clamped loads below contribute nothing
   if (a.norm) {
@@ -159,15 +174,21 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   for (int c = 0; c < NACC; ++c)
 #pragma unroll
     for (int t = 0; t < TT; ++t) acc[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int kk0 = wave * rpw;  // this wavefront's rows, relative to k_wg
-  if (have_col) {
+  if (have_first) {
     for (int kb = 0; kb < rpw && k_wg + kk0 + kb < K; kb += 8 * RPI) {
       f32x4 r[NACC][8];
+      if (kb == 0) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int row = min(k_wg + kk0 + kb + u * RPI + sub, K - 1);
+        for (int u = 0; u < 8; ++u)
 #pragma unroll
-        for (int c = 0; c < NACC; ++c) r[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+          for (int c = 0; c < NACC; ++c) r[c][u] = r_first[c][u];
+      } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int row = min(k_wg + kk0 + kb + u * RPI + sub, K - 1);
+#pragma unroll
+          for (int c = 0; c < NACC; ++c) r[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+        }
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u)
