@@ -296,6 +296,27 @@ def test_generate_greedy_on_device_matches_the_step_loop(hip):
         hip.LlamaModel(16, 8, 1, 1, 8).generate_greedy(3)     # no logits yet
 
 
+def test_long_generation_across_cache_growth_equals_one_prefill(hip):
+    # 1100 tokens generated on the device: the block caches grow 256 -> 512 -> 1024 -> 2048 while
+    # steps are queued.  Feeding the same 1103 tokens as one prompt to a fresh cache (prefill
+    # kernels, library GEMMs) must give the same next-token logits within the bar, and the same
+    # generation again the same ids and bits.
+    m, w = _tiny_model(hip)
+    toks = [1, 42, 100]
+    m.run(toks, want_logits=False)
+    got = m.generate_greedy(1100)
+    assert len(got) == 1100 and m.cache_len == 1103
+    last = m.logits()
+    m.clear_cache()
+    m.run(toks + got, want_logits=True)
+    rm.assert_close(m.logits(), last, 5 * ATOL, 5 * RTOL, "decode of 1100 tokens against one prefill of all of them")
+    m.clear_cache()
+    m.run(toks, want_logits=False)
+    again = m.generate_greedy(1100)
+    assert again == got
+    np.testing.assert_array_equal(m.logits(), last)
+
+
 # ---- the sampler on the device ---------------------------------------------------------------
 @pytest.fixture(scope="module")
 def sampler_model(hip):
