@@ -8,6 +8,7 @@
 #include <cstring>
 #include <array>
 #include <map>
+#include <mutex>
 #include <vector>
 
 #include "../../include/shainet_hip_attn.h"
@@ -36,7 +37,9 @@ struct RocBlas {
   rb_set_stream_t set_stream = nullptr;
   rb_sgemm_t sgemm = nullptr;
   bool tried = false;
+  std::mutex once;  // contexts on different threads may come here at the same time
   bool load() {
+    std::lock_guard<std::mutex> guard(once);
     if (tried) return sgemm != nullptr;
     tried = true;
     for (const char *name : {"librocblas.so.5", "librocblas.so"}) {
@@ -69,7 +72,9 @@ struct HipBlasLt {
   decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
   decltype(&hipblasLtMatmul) matmul = nullptr;
   bool tried = false, ok = false;
+  std::mutex once;
   bool load() {
+    std::lock_guard<std::mutex> guard(once);
     if (tried) return ok;
     tried = true;
     for (const char *name : {"libhipblaslt.so.1", "libhipblaslt.so"}) {
