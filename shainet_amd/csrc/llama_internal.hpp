@@ -74,7 +74,9 @@ struct Projector {
 
  private:
   int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
-  int gemm_lt(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
+  // res != nullptr: y = res + x W
+  int gemm_lt(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
+              const float *res = nullptr);
 };
 
 // Replace *dst (device, hipMalloc'ed or null) by a copy of n host floats.

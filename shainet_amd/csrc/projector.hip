@@ -171,7 +171,7 @@ void DevF::release() {
 
 // 1 = done, 0 = not available for this shape (the caller falls back to rocBLAS), < 0 = -status
 int Projector::gemm_lt(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N,
-                       hipStream_t stream) {
+                       hipStream_t stream, const float *res) {
   if (!g_lt.load()) return 0;
   if (!lt) {
     LtState *s = new LtState();
@@ -226,18 +226,25 @@ int Projector::gemm_lt(const float *x, long long x_stride, const float *w, float
     lt->workspace = np;
     lt->workspace_cap = sh.workspace;
   }
+  // res: y = res + x W in the library's epilogue (D = A B + C): one fp32 add per element, as in
+  // the separate add kernel
   const float one = 1.0f, zero = 0.0f;
-  const hipblasStatus_t st = g_lt.matmul(lt->handle, lt->desc, &one, w, sh.a, x, sh.b, &zero, y, sh.c, y, sh.c, &sh.algo,
-                                         lt->workspace, sh.workspace, stream);
+  const hipblasStatus_t st = g_lt.matmul(lt->handle, lt->desc, &one, w, sh.a, x, sh.b, res ? &one : &zero,
+                                         res ? res : y, sh.c, y, sh.c, &sh.algo, lt->workspace, sh.workspace, stream);
   return st == HIPBLAS_STATUS_SUCCESS ? 1 : -(int)st;
+}
+
+// hipBLASLt where its kernels are the faster ones on this device: many rows, or a large
+// weight matrix (rocBLAS picks slow kernels for long K with few rows)
+static bool wants_lt(int T, int K, int N) {
+  const int force = gemm_backend_override();
+  return force == 2 || (force == 0 && (T >= 256 || (long long)K * N > (8ll << 20)));
 }
 
 int Projector::gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N,
                     hipStream_t stream) {
-  // hipBLASLt where its kernels are the faster ones on this device: many rows, or a
-  // large weight matrix (rocBLAS picks slow kernels for long K with few rows)
   const int force = gemm_backend_override();
-  const bool want_lt = force == 2 || (force == 0 && (T >= 256 || (long long)K * N > (8ll << 20)));
+  const bool want_lt = wants_lt(T, K, N);
   if (want_lt) {
     const int r = gemm_lt(x, x_stride, w, y, T, K, N, stream);
     if (r == 1) return SHAINET_HIP_OK;
@@ -327,6 +334,11 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     if (rc) return rc;
     e = launch_swiglu_act(wide.p, y, T, N, stream);
   } else if (f.epilogue == kGemvResidual) {
+    if (f.res != y && wants_lt(T, K, N)) {  // the library adds the residual in its epilogue
+      const int r = gemm_lt(xin, xs, w, y, T, K, N, stream, f.res);
+      if (r == 1) return SHAINET_HIP_OK;
+      if (r < 0) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipblasLtMatmul failed with status " + std::to_string(-r));
+    }
     if (!wide.reserve((size_t)T * N)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
     int rc = gemm(xin, xs, w, wide.p, T, K, N, stream);
     if (rc) return rc;
