@@ -313,9 +313,11 @@ int shainet_hf_rope_freqs(const shainet_hf_llama_config *cfg, float *out, int n)
 int shainet_hf_load_llama(const char *model_dir, shainet_llama_model **out);
 
 /* Kernel timing for benchmarks: while enabled, every shainet_attn_forward call
- * brackets its attention kernel (the split-K decode kernel, the MFMA prefill
- * kernel or the generic kernel; not the prep or combine kernels) with HIP events
- * on the context's stream.  shainet_attn_profile_read waits for the stream,
+ * times its attention kernel (the split-K decode kernel, the MFMA prefill kernel
+ * with its combine kernel when it has one, or the generic kernel; not the prep
+ * kernel) with a pair of HIP events on the context's stream.  For the decode and
+ * prefill kernels the events take the kernel's own start and end clock readings
+ * (hipExtLaunchKernel), so the idle time between two kernels is not counted.  shainet_attn_profile_read waits for the stream,
  * returns the summed kernel time in milliseconds and the number of launches
  * since the last read, and resets both; shainet_attn_profile_samples does the same
  * but hands back the time of each launch (the first `capacity` of them; *launches

@@ -18,6 +18,8 @@
 // pieces of K rows.
 #include "attn_kernels.hpp"
 
+#include <hip/hip_ext.h>
+
 #include <math.h>
 #include <stdlib.h>
 
@@ -571,7 +573,7 @@ size_t prefill_partial_floats(const Shape &sh, int items, int ns) {
 
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                           const SeqTable &st, const Shape &sh, int items, int ns, float scale,
-                          hipStream_t stream, int wgs_per_cu) {
+                          hipStream_t stream, int wgs_per_cu, hipEvent_t before, hipEvent_t after) {
   if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1 || ns < 1 || (ns > 1 && !partials))
     return hipErrorInvalidValue;
   const long long n_wgs = (long long)items * sh.KV * ns;
@@ -600,11 +602,11 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
 #define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                    \
   do {                                                                                                          \
     if (groups == 2)                                                                                            \
-      hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, q_rot, kc, vc, out, \
-                         part_o, part_ml, st, sh, ns, c);                                                       \
+      hipExtLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, before,          \
+                            ns == 1 ? after : nullptr, 0, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);  \
     else                                                                                                        \
-      hipLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, q_rot, kc, vc, out, \
-                         part_o, part_ml, st, sh, ns, c);                                                       \
+      hipExtLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, before,          \
+                            ns == 1 ? after : nullptr, 0, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);  \
   } while (0)
   if (sh.hd == 64) {
     if (ns > 1)
@@ -620,8 +622,8 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
 #undef SHAINET_LAUNCH_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || ns == 1) return e;
-  hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, part_o, part_ml,
-                     out, st, sh, ns, c);
+  hipExtLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, nullptr,
+                        after, 0, part_o, part_ml, out, st, sh, ns, c);
   return hipGetLastError();
 }
 

@@ -60,13 +60,20 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 
 // q_rot: rotated queries [rows][H*hd]; the cache already holds the new rows.
-// pair_count: one zero-initialised int per (sequence, kv head); the kernel leaves it zero.
+// before / after (here and in launch_prefill; nullable): events that receive the first clock
+// reading of the first kernel and the last one of the last kernel of the launch.
+// part_flag: DecodePlan::n_slots words of device memory, zero when allocated and never reset;
+// epoch: a non-zero value no earlier launch on the same part_flag has used (the kernel marks
+// a finished partial with it); error: an int the device can write (pinned host memory will
+// do), set to 1 when a workgroup gave up waiting for the partials of others.
 struct DecodeArgs {
   const float *q_rot;
   const float *kc, *vc;
   float *out;
   float *partials;
-  int *pair_count;
+  unsigned *part_flag;
+  unsigned epoch;
+  int *error;
 };
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr);
@@ -79,7 +86,8 @@ size_t prefill_partial_floats(const Shape &sh, int items, int ns);
 // workgroups share a compute unit (a tuning knob).
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                           const SeqTable &st, const Shape &sh, int items, int ns, float scale,
-                          hipStream_t stream, int wgs_per_cu = 0);
+                          hipStream_t stream, int wgs_per_cu = 0, hipEvent_t before = nullptr,
+                          hipEvent_t after = nullptr);
 hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);

@@ -85,8 +85,12 @@ struct shainet_attn_ctx {
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
-  int *pair_count = nullptr;
-  size_t pair_count_cap = 0;
+  // decode split: a word per partial slot that says which launch completed it, the value
+  // the next launch uses, and a pinned host word the kernel sets when it gave up a wait
+  unsigned *part_flag = nullptr;
+  size_t part_flag_cap = 0;
+  unsigned decode_epoch = 0;
+  int *decode_error = nullptr;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
@@ -158,23 +162,33 @@ Shape shape_of(const shainet_attn_ctx *c, int cap) {
   return sh;
 }
 
-// Zero-initialised ints, one per (sequence, kv head), for the decode kernel's
-// last-arriver merge.  The kernel leaves them zero.
-int ensure_pair_counters(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
-  if (n <= c->pair_count_cap) return SHAINET_HIP_OK;
-  size_t want = c->pair_count_cap ? c->pair_count_cap : 256;
+// Zero-initialised words, one per partial slot of the decode split, and the error word.
+int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
+  if (!c->decode_error) {
+    HIP_TRY(hipHostMalloc((void **)&c->decode_error, sizeof(int), hipHostMallocDefault));
+    *c->decode_error = 0;
+  }
+  if (n <= c->part_flag_cap) return SHAINET_HIP_OK;
+  size_t want = c->part_flag_cap ? c->part_flag_cap : 1024;
   while (want < n) want *= 2;
-  int *np = nullptr;
-  HIP_TRY(hipMalloc((void **)&np, want * sizeof(int)));
-  hipError_t e = hipMemsetAsync(np, 0, want * sizeof(int), stream);
+  unsigned *np = nullptr;
+  HIP_TRY(hipMalloc((void **)&np, want * sizeof(unsigned)));
+  hipError_t e = hipMemsetAsync(np, 0, want * sizeof(unsigned), stream);
   if (e != hipSuccess) {
     (void)hipFree(np);
-    return hip_fail(e, "hipMemsetAsync(pair counters)");
+    return hip_fail(e, "hipMemsetAsync(partial flags)");
   }
-  if (c->pair_count) (void)hipFree(c->pair_count);  // hipFree waits for the device
-  c->pair_count = np;
-  c->pair_count_cap = want;
+  if (c->part_flag) (void)hipFree(c->part_flag);  // hipFree waits for the device
+  c->part_flag = np;
+  c->part_flag_cap = want;
   return SHAINET_HIP_OK;
+}
+
+// After a wait for the stream: did a decode launch give up waiting for partials?
+int check_decode_error(shainet_attn_ctx *c) {
+  if (!c->decode_error || *(volatile int *)c->decode_error == 0) return SHAINET_HIP_OK;
+  *c->decode_error = 0;
+  return fail(SHAINET_HIP_ERR_RUNTIME, "decode attention: partial results of other workgroups never arrived");
 }
 
 // Attention over a cache: shared by the fused entry point and by attention_kv_f32.
@@ -195,15 +209,18 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
   if (path == Path::kDecodeSplitK) {
     const DecodePlan plan = plan_decode(st, sh, c->decode_wgs_override);
     int rc = c->partials.reserve(decode_partial_floats(sh, plan));
-    if (!rc) rc = ensure_pair_counters(c, (size_t)st.n_seqs * sh.KV, stream);
+    if (!rc) rc = ensure_decode_flags(c, (size_t)plan.n_slots, stream);
     if (rc) return rc;
+    if (++c->decode_epoch == 0) c->decode_epoch = 1;  // zero is what untouched words hold
     DecodeArgs d;
     d.q_rot = q_rot;
     d.kc = kc;
     d.vc = vc;
     d.out = out;
     d.partials = c->partials.p;
-    d.pair_count = c->pair_count;
+    d.part_flag = c->part_flag;
+    d.epoch = c->decode_epoch;
+    d.error = c->decode_error;
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);
       if (e != hipSuccess) return hip_fail(e, "prep launch");
@@ -219,10 +236,8 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
       int ns = c->prefill_splits_override > 0 ? c->prefill_splits_override : prefill_key_splits(st, sh, items);
       int rc = c->partials.reserve(prefill_partial_floats(sh, items, ns));
       if (rc) return rc;
-      if (ev0) (void)hipEventRecord(ev0, stream);
       e = launch_prefill(q_rot, kc, vc, out, c->partials.p, st, sh, items, ns, scale, stream,
-                         c->prefill_wgs_per_cu);
-      if (ev1) (void)hipEventRecord(ev1, stream);
+                         c->prefill_wgs_per_cu, ev0, ev1);
     } else {
       plan_work(st, sh, path);
       if (ev0) (void)hipEventRecord(ev0, stream);
@@ -373,7 +388,8 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
   for (float *p : {c->d_q_norm, c->d_k_norm, c->d_bq, c->d_bk, c->d_bv})
     if (p) (void)hipFree(p);
   if (c->d_rope) (void)hipFree(c->d_rope);
-  if (c->pair_count) (void)hipFree(c->pair_count);
+  if (c->part_flag) (void)hipFree(c->part_flag);
+  if (c->decode_error) (void)hipHostFree(c->decode_error);
   for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
   delete c;
@@ -383,7 +399,7 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
 int shainet_attn_sync(shainet_attn_ctx *c) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
   HIP_TRY(hipStreamSynchronize(c->stream));
-  return SHAINET_HIP_OK;
+  return check_decode_error(c);
 }
 
 void *shainet_attn_stream(shainet_attn_ctx *c) { return c ? (void *)c->stream : nullptr; }
@@ -547,6 +563,10 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   if (!new_tokens || !q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (n_seqs < 1 || n_seqs > SHAINET_HIP_MAX_BATCH)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", SHAINET_HIP_MAX_BATCH);
+  if (mem == SHAINET_HIP_MEM_DEVICE &&
+      (q_stride < (long long)c->H * c->hd || k_stride < (long long)c->KV * c->hd || v_stride < (long long)c->KV * c->hd))
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "row strides must be at least the row widths %d and %d", c->H * c->hd,
+                c->KV * c->hd);
   SeqTable st;
   memset(&st, 0, sizeof st);
   st.n_seqs = n_seqs;
@@ -611,14 +631,15 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   pa.q_rot = c->q_rot.p;
   pa.kc = kc->k;
   pa.vc = kc->v;
+  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa);
+  if (rc) return rc;  // the cached lengths stay as they were: the call did not happen
   // the rows are in the cache once this call's kernels have run: @cache_len = total_len (llama_block.cr:288-289)
   for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
   c->last_rows = rows;
-  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa);
-  if (rc) return rc;
   if (mem == SHAINET_HIP_MEM_HOST) {
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
+    return check_decode_error(c);
   }
   return SHAINET_HIP_OK;
 }
@@ -664,9 +685,11 @@ int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int 
   st.n_new[0] = new_tokens;
   st.tok_off[1] = new_tokens;
   Shape sh = shape_of(c, kc->cap);
+  const int rc = run_attention(c, c->q_rot.p, kc->k, kc->v, out, st, sh, new_tokens, c->scale, c->stream, nullptr);
+  if (rc) return rc;
   kc->len[0] += new_tokens;
   c->last_rows = new_tokens;
-  return run_attention(c, c->q_rot.p, kc->k, kc->v, out, st, sh, new_tokens, c->scale, c->stream, nullptr);
+  return SHAINET_HIP_OK;
 }
 
 extern "C" {

@@ -10,9 +10,12 @@
 // sequence lengths are.  A span that crosses a pair boundary is processed as two
 // segments.  The four wavefronts of a workgroup take the tiles of a segment
 // round-robin, each keeping its own online softmax, and merge through LDS into
-// one partial (max, sum, O) per segment; the workgroup that delivers the last
-// partial of a pair (an atomic counter per pair tells) merges them and writes the
-// output row, so a decode step is one launch.
+// one partial (max, sum, O) per segment; the workgroup that holds the end of a
+// pair waits, once its own span is done, for the partials of the workgroups that
+// hold the pair's earlier parts (a word per partial says when it is complete),
+// merges them in a fixed order and writes the output row, so a decode step is one
+// launch.  Nothing a workgroup does between two segments waits for another
+// workgroup, and the next segment's first loads are in flight by then.
 //
 // Per 16-key tile a wavefront
 //   * copies the K tile (16 contiguous rows) from HBM straight into LDS with
@@ -35,6 +38,8 @@
 //           key 4*j + r of the tile, where accumulator register r of S^T lives.
 #include "attn_kernels.hpp"
 
+#include <hip/hip_ext.h>
+
 #include <math.h>
 #include <stdint.h>
 
@@ -49,8 +54,8 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Split-K partials cross workgroups that may sit on different XCDs, whose L2
 // caches are not kept coherent with each other for ordinary accesses.  Relaxed
 // atomic accesses at agent scope compile to write-through stores and cache-
-// bypassing loads, which is all that is needed for data published through an
-// atomic counter.
+// bypassing loads, which is all that is needed for data published through a
+// flag word written after them.
 __device__ __forceinline__ void coherent_store(float *p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -96,21 +101,49 @@ __device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last
   }
 }
 
+// One segment of a workgroup's span: tiles [tile0, tile1) of one (sequence, kv head) pair.
+struct Segment {
+  int s, kvh, L, n_s, tile0, tile1, token;
+  const float *kbase, *vbase;
+};
+
+// The segment that starts at tile t of the stream; s: a sequence at or before t's, moved up to it.
+__device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const SeqTable &st, const Shape &sh, int hd,
+                                              const float *kc, const float *vc) {
+  while (s + 1 < st.n_seqs && t >= st.work_off[s + 1]) ++s;
+  Segment g;
+  g.s = s;
+  g.L = st.start_pos[s] + 1;  // visible keys of the one new row
+  g.n_s = (g.L + 15) >> 4;    // tiles per kv head of this sequence
+  const int rel = t - st.work_off[s];
+  g.kvh = rel / g.n_s;
+  g.tile0 = rel - g.kvh * g.n_s;
+  g.tile1 = g.tile0 + min(g.n_s - g.tile0, t_end - t);
+  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)g.kvh * sh.cap * hd;
+  g.kbase = kc + head_base;
+  g.vbase = vc + head_base;
+  g.token = st.tok_off[s];
+  return g;
+}
+
+constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each
+
+// part_flag: one word per partial slot, never reset: a partial is complete when its word holds
+// this launch's `epoch` (the host hands out a new non-zero value per launch).  error: set when
+// the wait for other workgroups' partials was given up.
 template <int HD, int NW>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(const float *__restrict__ q_rot,
-                                                               const float *__restrict__ kc,
-                                                               const float *__restrict__ vc,
-                                                               float *__restrict__ out, float *part_o,
-                                                               float *part_ml, int *pair_count, SeqTable st,
-                                                               Shape sh, int tiles_per_wg, int total_tiles,
-                                                               int n_slots, float c) {
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
+    const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
+    float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned epoch, int *error,
+    SeqTable st, Shape sh, int tiles_per_wg, int total_tiles, int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
+  // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
+  // rows [g][HD] in its second one while the first already receives the next segment's tile
   __shared__ __attribute__((aligned(1024))) char k_lds[NW][2][C::TILE_BYTES];
-  // after its last tile a wavefront parks its O rows [g][HD] in its own K tile area
   __shared__ float sm_m[NW][16], sm_l[NW][16];  // per wavefront and head: running max, sum
-  __shared__ bool last_flag;
-  constexpr int WAVE_LDS_FLOATS = 2 * C::TILE_BYTES / 4;  // floats between two wavefronts' areas
+  constexpr int TILE_FLOATS = C::TILE_BYTES / 4;
+  constexpr int WAVE_LDS_FLOATS = 2 * TILE_FLOATS;  // floats between two wavefronts' areas
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, j = lane >> 4;
@@ -124,43 +157,44 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   // along them with dependent scalar loads took 2.5 us for a workgroup in the middle of 16
   // sequences).
   int s = (int)__popcll(__ballot(lane + 1 < st.n_seqs && t_begin >= st.work_off[lane + 1 < kMaxSeqs ? lane + 1 : kMaxSeqs]));
-  while (t < t_end) {
-    while (s + 1 < st.n_seqs && t >= st.work_off[s + 1]) ++s;
-    const int L = st.start_pos[s] + 1;  // visible keys of the one new row
-    const int n_s = (L + 15) >> 4;      // tiles per kv head of this sequence
-    const int rel = t - st.work_off[s];
-    const int kvh = rel / n_s, tile0 = rel - kvh * n_s;
-    const int seg_tiles = min(n_s - tile0, t_end - t);
-    const int tile1 = tile0 + seg_tiles;
-    const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
-    const float *kbase = kc + head_base;
-    const float *vbase = vc + head_base;
-    const int token = st.tok_off[s];
+  Segment seg = segment_at(t, t_end, s, st, sh, HD, kc, vc);
 
+  f32x4 v_next[4][C::NVU];
+  float qr[HD / 4];
+  // first tile of a segment into the wavefront's first buffer, its V rows and the query rows
+  auto start_segment = [&](const Segment &sg) {
+    const int tile = sg.tile0 + wave;
+    if (tile < sg.tile1) {
+      issue_k_tile<HD>(sg.kbase, tile * 16, sg.L - 1, my_lds, lane);
+      load_v_tile<HD>(sg.vbase, tile * 16, sg.L - 1, col, j, v_next);
+    }
+    const float *qp = q_rot + ((long long)sg.token * sh.H + sg.kvh * g + (col < g ? col : 0)) * HD + 4 * j;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      f32x4 x = *(const f32x4 *)(qp + 16 * i);
+      if (col >= g) x = f32x4{0.f, 0.f, 0.f, 0.f};
+      qr[4 * i + 0] = x.x;
+      qr[4 * i + 1] = x.y;
+      qr[4 * i + 2] = x.z;
+      qr[4 * i + 3] = x.w;
+    }
+  };
+  start_segment(seg);
+
+  // the pair whose last segment this workgroup holds without holding all of it: merged at the
+  // end of the span (only a span's first segment can start inside a pair, so there is one at most)
+  bool have_merge = false;
+  Segment mseg = seg;
+
+  for (;;) {
+    const int L = seg.L, tile1 = seg.tile1;
+    const float *kbase = seg.kbase, *vbase = seg.vbase;
     float m = -INFINITY, l = 0.f;
     f32x4 o[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    f32x4 v_next[4][C::NVU];
-    int tile = tile0 + wave;
-    float qr[HD / 4];
-    if (tile < tile1) {
-      issue_k_tile<HD>(kbase, tile * 16, L - 1, my_lds, lane);
-      load_v_tile<HD>(vbase, tile * 16, L - 1, col, j, v_next);
-    }
-    {
-      const float *qp = q_rot + ((long long)token * sh.H + kvh * g + (col < g ? col : 0)) * HD + 4 * j;
-#pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        f32x4 x = *(const f32x4 *)(qp + 16 * i);
-        if (col >= g) x = f32x4{0.f, 0.f, 0.f, 0.f};
-        qr[4 * i + 0] = x.x;
-        qr[4 * i + 1] = x.y;
-        qr[4 * i + 2] = x.z;
-        qr[4 * i + 3] = x.w;
-      }
-    }
+    int tile = seg.tile0 + wave;
     for (int it = 0; tile < tile1; tile += NW, ++it) {
       const int kb = tile * 16;
       char *buf = my_lds + (it & 1) * C::TILE_BYTES;
@@ -215,11 +249,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         }
     }
 
-    // merge the wavefronts through LDS: each one's tiles are consumed, so its K tile
-    // area is free to hold its O rows
+    // merge the wavefronts through LDS: each one's tiles are consumed, so its second K tile
+    // buffer is free to hold its O rows
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    float *sm_o = (float *)&k_lds[0][0][0];
+    float *sm_o = (float *)&k_lds[0][1][0];
     if (col < g) {
       float *dst = sm_o + wave * WAVE_LDS_FLOATS + col * HD;
 #pragma unroll
@@ -232,8 +266,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       }
     }
     __syncthreads();
-    const bool whole_pair = tile0 == 0 && tile1 == n_s;
-    const int pair = s * sh.KV + kvh;
+    const bool whole_pair = seg.tile0 == 0 && tile1 == seg.n_s;
+    const int pair = seg.s * sh.KV + seg.kvh;
     const int slot = blockIdx.x + pair;  // unique: both terms only grow along the tile stream
     for (int idx = threadIdx.x; idx < g * HD; idx += 64 * NW) {
       const int cc = idx / HD, d = idx - cc * HD;
@@ -248,7 +282,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         ls += f * sm_l[w][cc];
       }
       if (whole_pair) {
-        out[((long long)token * sh.H + kvh * g + cc) * HD + d] = acc / ls;
+        out[((long long)seg.token * sh.H + seg.kvh * g + cc) * HD + d] = acc / ls;
       } else if (slot < n_slots) {
         const long long pi = (long long)slot * g + cc;
         coherent_store(&part_o[pi * HD + d], acc);
@@ -258,74 +292,97 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         }
       }
     }
-    // Every wavefront is done with the O rows parked in LDS (the next segment's K
-    // tiles land there).  Partials are written through to device-coherent memory
-    // (coherent_store); each wavefront waits for its stores to be acknowledged
-    // (s_waitcnt vmcnt(0): the barrier alone does not) before the arrival is counted.
+    if (!whole_pair && tile1 == seg.n_s) {
+      have_merge = true;
+      mseg = seg;
+    }
+    // The next segment's first loads go out before this one's partial is published: the wait
+    // below covers both.  (Its K tile lands in the wavefront's first buffer, which only this
+    // wavefront reads; the parked rows are in the second ones.)
+    t += tile1 - seg.tile0;
+    const bool more = t < t_end;
+    if (more) {
+      seg = segment_at(t, t_end, s, st, sh, HD, kc, vc);
+      start_segment(seg);
+    }
+    // Partials are written through to device-coherent memory (coherent_store); each wavefront
+    // waits for its stores to be acknowledged (s_waitcnt vmcnt(0): the barrier alone does not),
+    // then one lane marks the partial complete.  The barrier also ends the reads of the parked rows.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (!whole_pair) {
-      // The last workgroup to deliver a partial of this pair merges them all.  The
-      // counter returns to zero for the next launch.
-      const int a = st.work_off[s] + kvh * n_s;  // the pair's tiles are [a, a + n_s)
-      const int w_lo = a / tiles_per_wg, w_hi = (a + n_s - 1) / tiles_per_wg;
-      const int n_part = w_hi - w_lo + 1;
-      if (threadIdx.x == 0) {
-        const int old = atomicAdd(&pair_count[pair], 1);
-        last_flag = old == n_part - 1;
-        if (last_flag) atomicExch(&pair_count[pair], 0);
-      }
-      __syncthreads();
-      if (last_flag) {
-        // every partial of the pair is in memory: drop whatever this XCD's caches
-        // still hold of those addresses, then read them with ordinary wide loads
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        constexpr int LPR = HD / 4;       // lanes that cover one row with float4
-        constexpr int GROUPS = 64 / LPR;  // partials handled side by side
-        const int d4 = lane % LPR, grp = lane / LPR;
-        const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
-        for (int cc = wave; cc < g; cc += NW) {
-          const long long first = base + cc;
-          float mm = -INFINITY;
-          for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
-          for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
-          float ls = 0.f;
-          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-          for (int i0 = 0; i0 < n_part; i0 += 8 * GROUPS) {  // eight rows in flight per lane
-            f32x4 x[8];
-            float f[8], lp[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-              const int i = i0 + u * GROUPS + grp;
-              const long long pi = first + (long long)min(i, n_part - 1) * g;
-              x[u] = *(const f32x4 *)&part_o[pi * HD + 4 * d4];
-              f[u] = part_ml[2 * pi];
-              lp[u] = part_ml[2 * pi + 1];
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-              const int i = i0 + u * GROUPS + grp;
-              const float w = i < n_part ? fast_exp2((f[u] - mm) * c) : 0.f;
-              acc += w * x[u];
-              ls += w * lp[u];
-            }
-          }
-#pragma unroll
-          for (int o2 = LPR; o2 < 64; o2 <<= 1) {
-            acc.x += __shfl_xor(acc.x, o2);
-            acc.y += __shfl_xor(acc.y, o2);
-            acc.z += __shfl_xor(acc.z, o2);
-            acc.w += __shfl_xor(acc.w, o2);
-            ls += __shfl_xor(ls, o2);
-          }
-          if (grp == 0) {
-            const float inv = 1.0f / ls;
-            *(f32x4 *)&out[((long long)token * sh.H + kvh * g + cc) * HD + 4 * d4] = acc * inv;
-          }
+    if (!whole_pair && threadIdx.x == 0 && slot < n_slots)
+      __hip_atomic_store(&part_flag[slot], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!more) break;
+  }
+
+  if (have_merge) {
+    // This workgroup holds the end of a pair that others began: they have lower indices, were
+    // started before this one and wait for nobody, so waiting for their partials is safe.
+    const int a = st.work_off[mseg.s] + mseg.kvh * mseg.n_s;  // the pair's tiles are [a, a + n_s)
+    const int w_lo = a / tiles_per_wg;
+    const int n_part = (int)blockIdx.x - w_lo + 1;
+    const int pair = mseg.s * sh.KV + mseg.kvh;
+    if (wave == 0) {
+      const unsigned *fl = part_flag + w_lo + pair;
+      for (int spins = 0;; ++spins) {
+        bool ok = true;
+        for (int i = lane; i < n_part; i += 64)
+          ok = ok && __hip_atomic_load(fl + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == epoch;
+        if (__all(ok)) break;
+        if (spins >= kFlagSpinLimit) {
+          if (lane == 0) *error = 1;
+          break;
         }
+        __builtin_amdgcn_s_sleep(2);
       }
     }
-    t += seg_tiles;
+    __syncthreads();
+    // every partial of the pair is in memory: drop whatever this XCD's caches
+    // still hold of those addresses, then read them with ordinary wide loads
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    constexpr int LPR = HD / 4;       // lanes that cover one row with float4
+    constexpr int GROUPS = 64 / LPR;  // partials handled side by side
+    const int d4 = lane % LPR, grp = lane / LPR;
+    const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
+    for (int cc = wave; cc < g; cc += NW) {
+      const long long first = base + cc;
+      float mm = -INFINITY;
+      for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
+      for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
+      float ls = 0.f;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int i0 = 0; i0 < n_part; i0 += 8 * GROUPS) {  // eight rows in flight per lane
+        f32x4 x[8];
+        float f[8], lp[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u * GROUPS + grp;
+          const long long pi = first + (long long)min(i, n_part - 1) * g;
+          x[u] = *(const f32x4 *)&part_o[pi * HD + 4 * d4];
+          f[u] = part_ml[2 * pi];
+          lp[u] = part_ml[2 * pi + 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u * GROUPS + grp;
+          const float w = i < n_part ? fast_exp2((f[u] - mm) * c) : 0.f;
+          acc += w * x[u];
+          ls += w * lp[u];
+        }
+      }
+#pragma unroll
+      for (int o2 = LPR; o2 < 64; o2 <<= 1) {
+        acc.x += __shfl_xor(acc.x, o2);
+        acc.y += __shfl_xor(acc.y, o2);
+        acc.z += __shfl_xor(acc.z, o2);
+        acc.w += __shfl_xor(acc.w, o2);
+        ls += __shfl_xor(ls, o2);
+      }
+      if (grp == 0) {
+        const float inv = 1.0f / ls;
+        *(f32x4 *)&out[((long long)mseg.token * sh.H + mseg.kvh * g + cc) * HD + 4 * d4] = acc * inv;
+      }
+    }
   }
 }
 
@@ -361,7 +418,8 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before, hipEvent_t after) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
-      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.pair_count)
+      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.part_flag || !d.error ||
+      d.epoch == 0)
     return hipErrorInvalidValue;
   for (int s = 0; s < st.n_seqs; ++s)
     if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
@@ -370,16 +428,20 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   float *part_o = d.partials;
   float *part_ml = d.partials + (size_t)p.n_slots * sh.g * sh.hd;
   const float c = scale * kLog2e;
-  if (before) (void)hipEventRecord(before, stream);
+  // before / after (nullable) receive the kernel's own first and last clock reading, not the
+  // time at which the stream reached them: what is between two kernels stays out
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
-    hipLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, d.q_rot, d.kc, d.vc, d.out,
-                       part_o, part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.epoch, d.error, st, sh, p.tiles_per_wg,
+                          p.total_tiles,
+                          p.n_slots, c);
   else
-    hipLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, d.q_rot, d.kc, d.vc, d.out,
-                       part_o, part_ml, d.pair_count, st, sh, p.tiles_per_wg, p.total_tiles, p.n_slots, c);
+    hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.epoch, d.error, st, sh, p.tiles_per_wg,
+                          p.total_tiles,
+                          p.n_slots, c);
   hipError_t e = hipGetLastError();
-  if (after) (void)hipEventRecord(after, stream);
   return e;
 }
 
