@@ -119,7 +119,9 @@ struct GemvArgs {
   const float *res;      // kGemvResidual: [T, N], y = res + x W
   float *y;              // [T, N]; kGemvSwiglu: silu(x W_gate) * (x W_up)
   float *partials;       // GemvPlan::partial_floats floats when the plan has splits > 1
-  int *counters;         // GemvPlan::col_tiles zero-initialised ints, left zero
+  unsigned *flags;       // GemvPlan::col_tiles * splits words, zero when allocated and never reset
+  unsigned epoch;        // non-zero, used by no earlier launch on the same flags
+  int *error;            // device-writable int, set to 1 when a wait for partials was given up
   int T, K, N;
   int epilogue;
   int rows_per_wave;     // filled in by launch_gemv
@@ -135,6 +137,12 @@ struct GemvPlan {
 // head_dim: kGemvQkvPrep only (a column tile must hold whole heads)
 GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim = 0);
 hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
+
+// One pinned host int for the whole library that kernels set when they give up a bounded
+// wait for other workgroups (null when it cannot be allocated); check_error_word, called
+// after a wait for a stream, turns a set word into SHAINET_HIP_ERR_RUNTIME and clears it.
+int *error_word();
+int check_error_word();
 
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
                                 int num_kv_heads, int head_dim, int capacity, hipStream_t stream);

@@ -31,6 +31,30 @@ int fail(int code, const char *fmt, ...) {
 // for the other translation units of the library
 void shainet_hip_set_error(int code, const char *msg) { fail(code, "%s", msg); }
 
+namespace shainet {
+
+int *error_word() {
+  static int *word = [] {
+    int *p = nullptr;
+    if (hipHostMalloc((void **)&p, sizeof(int), hipHostMallocPortable) != hipSuccess) {
+      (void)hipGetLastError();
+      return (int *)nullptr;
+    }
+    *p = 0;
+    return p;
+  }();
+  return word;
+}
+
+int check_error_word() {
+  int *w = error_word();
+  if (!w || *(volatile int *)w == 0) return SHAINET_HIP_OK;
+  *(volatile int *)w = 0;
+  return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups");
+}
+
+}  // namespace shainet
+
 namespace {
 
 int hip_fail(hipError_t e, const char *what) {
@@ -85,12 +109,11 @@ struct shainet_attn_ctx {
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
-  // decode split: a word per partial slot that says which launch completed it, the value
-  // the next launch uses, and a pinned host word the kernel sets when it gave up a wait
+  // decode split: a word per partial slot that says which launch completed it, and the value
+  // the next launch uses
   unsigned *part_flag = nullptr;
   size_t part_flag_cap = 0;
   unsigned decode_epoch = 0;
-  int *decode_error = nullptr;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
@@ -162,12 +185,9 @@ Shape shape_of(const shainet_attn_ctx *c, int cap) {
   return sh;
 }
 
-// Zero-initialised words, one per partial slot of the decode split, and the error word.
+// Zero-initialised words, one per partial slot of the decode split.
 int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
-  if (!c->decode_error) {
-    HIP_TRY(hipHostMalloc((void **)&c->decode_error, sizeof(int), hipHostMallocDefault));
-    *c->decode_error = 0;
-  }
+  if (!error_word()) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
   if (n <= c->part_flag_cap) return SHAINET_HIP_OK;
   size_t want = c->part_flag_cap ? c->part_flag_cap : 1024;
   while (want < n) want *= 2;
@@ -182,13 +202,6 @@ int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
   c->part_flag = np;
   c->part_flag_cap = want;
   return SHAINET_HIP_OK;
-}
-
-// After a wait for the stream: did a decode launch give up waiting for partials?
-int check_decode_error(shainet_attn_ctx *c) {
-  if (!c->decode_error || *(volatile int *)c->decode_error == 0) return SHAINET_HIP_OK;
-  *c->decode_error = 0;
-  return fail(SHAINET_HIP_ERR_RUNTIME, "decode attention: partial results of other workgroups never arrived");
 }
 
 // Attention over a cache: shared by the fused entry point and by attention_kv_f32.
@@ -220,7 +233,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     d.partials = c->partials.p;
     d.part_flag = c->part_flag;
     d.epoch = c->decode_epoch;
-    d.error = c->decode_error;
+    d.error = error_word();
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);
       if (e != hipSuccess) return hip_fail(e, "prep launch");
@@ -389,7 +402,6 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
     if (p) (void)hipFree(p);
   if (c->d_rope) (void)hipFree(c->d_rope);
   if (c->part_flag) (void)hipFree(c->part_flag);
-  if (c->decode_error) (void)hipHostFree(c->decode_error);
   for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
   delete c;
@@ -399,7 +411,7 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
 int shainet_attn_sync(shainet_attn_ctx *c) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
   HIP_TRY(hipStreamSynchronize(c->stream));
-  return check_decode_error(c);
+  return check_error_word();
 }
 
 void *shainet_attn_stream(shainet_attn_ctx *c) { return c ? (void *)c->stream : nullptr; }
@@ -639,7 +651,7 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   if (mem == SHAINET_HIP_MEM_HOST) {
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
-    return check_decode_error(c);
+    return check_error_word();
   }
   return SHAINET_HIP_OK;
 }

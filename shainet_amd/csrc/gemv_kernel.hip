@@ -6,10 +6,10 @@
 // well as along N to put enough workgroups in flight: a wavefront owns 256
 // consecutive columns (one float4 per lane, 1 KiB per W row) and a run of rows of
 // W; the four wavefronts of a workgroup take four runs and add up through LDS.
-// With more than one workgroup along K, each leaves a partial sum and the last one
-// to arrive at a column tile (an atomic counter per tile tells) adds the partials
-// in a fixed order, so results do not depend on scheduling, and applies the
-// epilogue.  Everything a decode step does around a product rides along:
+// With more than one workgroup along K, each leaves a partial sum and marks it
+// complete in a flag word; the last workgroup along K of a column tile waits for
+// the flags of the others, adds the partials in a fixed order, so results do not
+// depend on scheduling, and applies the epilogue.  Everything a decode step does around a product rides along:
 //   * prologue: RMSNorm of the x rows (rms_norm.cr:18-37, fp64 as there), so the
 //     normalised activations never go to memory;
 //   * epilogue: residual add (simple_matrix.cr:39-48), the SwiGLU gate
@@ -108,7 +108,6 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   extern __shared__ float smem[];  // xs[TT][4 * rows_per_wave]; reused for the cross-wavefront sums
   __shared__ double rms_s[TT];
   __shared__ double red_s[4];
-  __shared__ bool last_flag;
   __shared__ __align__(16) float tile_s[PREP ? 256 : 4];  // PREP: one finished row of this column tile
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int cl = lane % LPR, sub = lane / LPR;
@@ -259,18 +258,32 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
       }
   }
 
-  // ---- the last workgroup of this column tile adds the partials in a fixed order
-  // the partial stores above are acknowledged (s_waitcnt vmcnt(0): the barrier alone does
-  // not wait for them) before the arrival is counted
+  // ---- the last workgroup along K of this column tile adds the partials in a fixed order.
+  // The partial stores above are acknowledged (s_waitcnt vmcnt(0): the barrier alone does
+  // not wait for them) before the partial is marked complete.  The flag words are never
+  // reset: complete means holding this launch's epoch.
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int old = atomicAdd(&a.counters[blockIdx.x], 1);
-    last_flag = old == splits - 1;
-    if (last_flag) atomicExch(&a.counters[blockIdx.x], 0);  // ready for the next launch
+  unsigned *flags = a.flags + (long long)blockIdx.x * splits;
+  if ((int)blockIdx.y != splits - 1) {
+    if (threadIdx.x == 0) __hip_atomic_store(flags + blockIdx.y, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
+  // the others have lower indices, were started before this workgroup and wait for nobody
+  if (wave == 0) {
+    for (int spins = 0;; ++spins) {
+      bool ok = true;
+      for (int i = lane; i < splits - 1; i += 64)
+        ok = ok && __hip_atomic_load(flags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
+      if (__all(ok)) break;
+      if (spins >= (1 << 21)) {  // seconds
+        if (lane == 0) *a.error = 1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
   }
   __syncthreads();
-  if (!last_flag) return;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   for (int t = 0; t < T; ++t) {
     // row group g = wave * RPI + sub adds splits g, g + 4 * RPI, ... (FL loads in flight);
@@ -371,7 +384,7 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
   if (!a.y && a.epilogue != kGemvQkvPrep) return hipErrorInvalidValue;
   if (p.rows_per_instr != 1 && p.rows_per_instr != 4) return hipErrorInvalidValue;
   if (p.rows_per_wave < 8 * p.rows_per_instr || p.rows_per_wave % (8 * p.rows_per_instr)) return hipErrorInvalidValue;
-  if (p.splits > 1 && (!a.partials || !a.counters)) return hipErrorInvalidValue;
+  if (p.splits > 1 && (!a.partials || !a.flags || !a.error || a.epoch == 0)) return hipErrorInvalidValue;
   if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
   if (a.epilogue != kGemvResidual) a.res = nullptr;
   const bool prep = a.epilogue == kGemvQkvPrep;

@@ -262,7 +262,7 @@ static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_toke
   if (hipMemcpyAsync(out, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
-  return SHAINET_HIP_OK;
+  return check_error_word();
 }
 
 }  // extern "C"
@@ -449,7 +449,7 @@ static int block_forward_any(shainet_llama_block *b, const float *x, int new_tok
   if (hipMemcpyAsync(out, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
-  return SHAINET_HIP_OK;
+  return check_error_word();
 }
 
 }  // extern "C"

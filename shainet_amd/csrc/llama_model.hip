@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "../../include/shainet_hip_attn.h"
+#include "attn_kernels.hpp"
 #include "block_kernels.hpp"
 #include "llama_internal.hpp"
 
@@ -109,6 +110,7 @@ int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *v
       (vals && hipMemcpyAsync(vals, m->d_vals, k * sizeof(float), hipMemcpyDeviceToHost, m->stream) != hipSuccess) ||
       hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the selection back failed");
+  if (int rc = check_error_word()) return rc;
   *count = host_ids[kMaxTopK];
   for (int i = 0; i < k; ++i) ids[i] = host_ids[i];
   return SHAINET_HIP_OK;
@@ -251,6 +253,7 @@ int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tok
             hipSuccess ||
         hipStreamSynchronize(m->stream) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
+    return check_error_word();
   }
   return SHAINET_HIP_OK;
 }
@@ -287,6 +290,7 @@ int shainet_llama_model_generate_greedy(shainet_llama_model *m, int max_tokens, 
     if (hipMemcpyAsync(host_ids, m->d_gen, steps * sizeof(int), hipMemcpyDeviceToHost, m->stream) != hipSuccess ||
         hipStreamSynchronize(m->stream) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "copying the generated ids back failed");
+    if (int rc = check_error_word()) return rc;
     for (int i = 0; i < steps; ++i) {
       bool stop = false;
       for (int j = 0; j < n_stop; ++j) stop = stop || host_ids[i] == stop_ids[j];
@@ -309,7 +313,7 @@ int shainet_llama_model_sync(shainet_llama_model *m) {
   if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
   if (m->stream && hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamSynchronize failed");
-  return SHAINET_HIP_OK;
+  return check_error_word();
 }
 
 int shainet_llama_model_greedy(shainet_llama_model *m, int *token) {
@@ -360,7 +364,7 @@ int shainet_llama_model_read_logits(shainet_llama_model *m, float *logits) {
           hipSuccess ||
       hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
-  return SHAINET_HIP_OK;
+  return check_error_word();
 }
 
 }  // extern "C"

@@ -283,19 +283,22 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     }
     const GemvPlan p = plan_gemv(T, K, N, f.epilogue, f.prep ? f.prep->hd : 0);
     if (!scratch.reserve(p.partial_floats)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-    if ((size_t)p.col_tiles > counters_cap) {
-      size_t want = counters_cap ? counters_cap : 1024;
-      while (want < (size_t)p.col_tiles) want *= 2;
-      int *np = nullptr;
-      if (hipMalloc((void **)&np, want * sizeof(int)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-      if (hipMemsetAsync(np, 0, want * sizeof(int), stream) != hipSuccess) {
+    const size_t n_flags = (size_t)p.col_tiles * p.splits;
+    if (p.splits > 1 && n_flags > flags_cap) {
+      size_t want = flags_cap ? flags_cap : 4096;
+      while (want < n_flags) want *= 2;
+      unsigned *np = nullptr;
+      if (hipMalloc((void **)&np, want * sizeof(unsigned)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+      if (hipMemsetAsync(np, 0, want * sizeof(unsigned), stream) != hipSuccess) {
         (void)hipFree(np);
-        return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipMemsetAsync(counters) failed");
+        return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipMemsetAsync(flags) failed");
       }
-      if (counters) (void)hipFree(counters);  // hipFree waits for the device
-      counters = np;
-      counters_cap = want;
+      if (flags) (void)hipFree(flags);  // hipFree waits for the device
+      flags = np;
+      flags_cap = want;
     }
+    if (p.splits > 1 && !error_word()) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+    if (++epoch == 0) epoch = 1;  // zero is what untouched flag words hold
     GemvArgs a = {};
     a.x = xin;
     a.x_stride = xs;
@@ -306,7 +309,9 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.res = f.res;
     a.y = y;
     a.partials = scratch.p;
-    a.counters = counters;
+    a.flags = flags;
+    a.epoch = epoch;
+    a.error = error_word();
     a.T = T;
     a.K = K;
     a.N = N;
@@ -366,9 +371,9 @@ void Projector::release() {
   scratch.release();
   normed.release();
   wide.release();
-  if (counters) (void)hipFree(counters);
-  counters = nullptr;
-  counters_cap = 0;
+  if (flags) (void)hipFree(flags);
+  flags = nullptr;
+  flags_cap = 0;
 }
 
 int upload_floats(float **dst, const float *src, size_t n) {
