@@ -62,17 +62,15 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 // q_rot: rotated queries [rows][H*hd]; the cache already holds the new rows.
 // before / after (here and in launch_prefill; nullable): events that receive the first clock
 // reading of the first kernel and the last one of the last kernel of the launch.
-// part_flag: DecodePlan::n_slots words of device memory, zero when allocated and never reset;
-// epoch: a non-zero value no earlier launch on the same part_flag has used (the kernel marks
-// a finished partial with it); error: an int the device can write (pinned host memory will
-// do), set to 1 when a workgroup gave up waiting for the partials of others.
+// part_flag: DecodePlan::n_slots words of device memory, zero when allocated; the kernel
+// leaves them zero.  error: an int the device can write (pinned host memory will do), set
+// to 1 when a workgroup gave up waiting for the partials of others.
 struct DecodeArgs {
   const float *q_rot;
   const float *kc, *vc;
   float *out;
   float *partials;
   unsigned *part_flag;
-  unsigned epoch;
   int *error;
 };
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
@@ -119,8 +117,7 @@ struct GemvArgs {
   const float *res;      // kGemvResidual: [T, N], y = res + x W
   float *y;              // [T, N]; kGemvSwiglu: silu(x W_gate) * (x W_up)
   float *partials;       // GemvPlan::partial_floats floats when the plan has splits > 1
-  unsigned *flags;       // GemvPlan::col_tiles * splits words, zero when allocated and never reset
-  unsigned epoch;        // non-zero, used by no earlier launch on the same flags
+  unsigned *flags;       // GemvPlan::col_tiles * splits words, zero when allocated; left zero
   int *error;            // device-writable int, set to 1 when a wait for partials was given up
   int T, K, N;
   int epilogue;

@@ -50,7 +50,7 @@ int check_error_word() {
   int *w = error_word();
   if (!w || *(volatile int *)w == 0) return SHAINET_HIP_OK;
   *(volatile int *)w = 0;
-  return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups");
+  return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups; the results of the calls since the last wait are invalid and their contexts must be destroyed");
 }
 
 }  // namespace shainet
@@ -109,11 +109,9 @@ struct shainet_attn_ctx {
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
-  // decode split: a word per partial slot that says which launch completed it, and the value
-  // the next launch uses
+  // decode split: a word per partial slot that says when it is complete (zero between launches)
   unsigned *part_flag = nullptr;
   size_t part_flag_cap = 0;
-  unsigned decode_epoch = 0;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
@@ -224,7 +222,6 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     int rc = c->partials.reserve(decode_partial_floats(sh, plan));
     if (!rc) rc = ensure_decode_flags(c, (size_t)plan.n_slots, stream);
     if (rc) return rc;
-    if (++c->decode_epoch == 0) c->decode_epoch = 1;  // zero is what untouched words hold
     DecodeArgs d;
     d.q_rot = q_rot;
     d.kc = kc;
@@ -232,7 +229,6 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     d.out = out;
     d.partials = c->partials.p;
     d.part_flag = c->part_flag;
-    d.epoch = c->decode_epoch;
     d.error = error_word();
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);

@@ -12,7 +12,8 @@
 // round-robin, each keeping its own online softmax, and merge through LDS into
 // one partial (max, sum, O) per segment; the workgroup that holds the end of a
 // pair waits, once its own span is done, for the partials of the workgroups that
-// hold the pair's earlier parts (a word per partial says when it is complete),
+// hold the pair's earlier parts (a word per partial says when it is complete; the
+// merging workgroup clears it again),
 // merges them in a fixed order and writes the output row, so a decode step is one
 // launch.  Nothing a workgroup does between two segments waits for another
 // workgroup, and the next segment's first loads are in flight by then.
@@ -128,13 +129,14 @@ __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const Se
 
 constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each
 
-// part_flag: one word per partial slot, never reset: a partial is complete when its word holds
-// this launch's `epoch` (the host hands out a new non-zero value per launch).  error: set when
-// the wait for other workgroups' partials was given up.
+// part_flag: one word per partial slot, zero between launches: a workgroup sets the word of a
+// partial it has completed, the workgroup that merges the pair clears the words it waited for
+// (so a launch may be replayed as it is).  error: set when the wait for other workgroups'
+// partials was given up.
 template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
-    float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned epoch, int *error,
+    float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, int *error,
     SeqTable st, Shape sh, int tiles_per_wg, int total_tiles, int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
@@ -292,7 +294,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         }
       }
     }
-    if (!whole_pair && tile1 == seg.n_s) {
+    const bool pair_end = !whole_pair && tile1 == seg.n_s;
+    if (pair_end) {
       have_merge = true;
       mseg = seg;
     }
@@ -310,8 +313,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     // then one lane marks the partial complete.  The barrier also ends the reads of the parked rows.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (!whole_pair && threadIdx.x == 0 && slot < n_slots)
-      __hip_atomic_store(&part_flag[slot], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!whole_pair && !pair_end && threadIdx.x == 0 && slot < n_slots)
+      __hip_atomic_store(&part_flag[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (!more) break;
   }
 
@@ -323,12 +326,16 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const int n_part = (int)blockIdx.x - w_lo + 1;
     const int pair = mseg.s * sh.KV + mseg.kvh;
     if (wave == 0) {
-      const unsigned *fl = part_flag + w_lo + pair;
+      unsigned *fl = part_flag + w_lo + pair;  // the last of the n_part partials is this workgroup's own
       for (int spins = 0;; ++spins) {
         bool ok = true;
-        for (int i = lane; i < n_part; i += 64)
-          ok = ok && __hip_atomic_load(fl + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == epoch;
-        if (__all(ok)) break;
+        for (int i = lane; i < n_part - 1; i += 64)
+          ok = ok && __hip_atomic_load(fl + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+        if (__all(ok)) {
+          for (int i = lane; i < n_part - 1; i += 64)
+            __hip_atomic_store(fl + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
         if (spins >= kFlagSpinLimit) {
           if (lane == 0) *error = 1;
           break;
@@ -418,8 +425,7 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before, hipEvent_t after) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
-      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.part_flag || !d.error ||
-      d.epoch == 0)
+      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.part_flag || !d.error)
     return hipErrorInvalidValue;
   for (int s = 0; s < st.n_seqs; ++s)
     if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
@@ -433,12 +439,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
     hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.epoch, d.error, st, sh, p.tiles_per_wg,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg,
                           p.total_tiles,
                           p.n_slots, c);
   else
     hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.epoch, d.error, st, sh, p.tiles_per_wg,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg,
                           p.total_tiles,
                           p.n_slots, c);
   hipError_t e = hipGetLastError();

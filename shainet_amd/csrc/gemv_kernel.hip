@@ -260,13 +260,13 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 
   // ---- the last workgroup along K of this column tile adds the partials in a fixed order.
   // The partial stores above are acknowledged (s_waitcnt vmcnt(0): the barrier alone does
-  // not wait for them) before the partial is marked complete.  The flag words are never
-  // reset: complete means holding this launch's epoch.
+  // not wait for them) before the partial is marked complete in its flag word; the merging
+  // workgroup clears the words it waited for, so they are zero between launches.
   __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
   unsigned *flags = a.flags + (long long)blockIdx.x * splits;
   if ((int)blockIdx.y != splits - 1) {
-    if (threadIdx.x == 0) __hip_atomic_store(flags + blockIdx.y, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_store(flags + blockIdx.y, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   // the others have lower indices, were started before this workgroup and wait for nobody
@@ -274,8 +274,12 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
     for (int spins = 0;; ++spins) {
       bool ok = true;
       for (int i = lane; i < splits - 1; i += 64)
-        ok = ok && __hip_atomic_load(flags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
-      if (__all(ok)) break;
+        ok = ok && __hip_atomic_load(flags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+      if (__all(ok)) {
+        for (int i = lane; i < splits - 1; i += 64)
+          __hip_atomic_store(flags + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
       if (spins >= (1 << 21)) {  // seconds
         if (lane == 0) *a.error = 1;
         break;
@@ -384,7 +388,7 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
   if (!a.y && a.epilogue != kGemvQkvPrep) return hipErrorInvalidValue;
   if (p.rows_per_instr != 1 && p.rows_per_instr != 4) return hipErrorInvalidValue;
   if (p.rows_per_wave < 8 * p.rows_per_instr || p.rows_per_wave % (8 * p.rows_per_instr)) return hipErrorInvalidValue;
-  if (p.splits > 1 && (!a.partials || !a.flags || !a.error || a.epoch == 0)) return hipErrorInvalidValue;
+  if (p.splits > 1 && (!a.partials || !a.flags || !a.error)) return hipErrorInvalidValue;
   if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
   if (a.epilogue != kGemvResidual) a.res = nullptr;
   const bool prep = a.epilogue == kGemvQkvPrep;

@@ -65,10 +65,9 @@ struct Projector {
   LtState *lt = nullptr;
   bool lt_broken = false;
   DevF scratch, normed, wide;
-  // split products: a word per partial that says which launch completed it; the next launch's value
+  // split products: a word per partial that says when it is complete (zero between launches)
   unsigned *flags = nullptr;
   size_t flags_cap = 0;
-  unsigned epoch = 0;
   // returns a SHAINET_HIP_* status; the message is left for shainet_hip_last_error
   int project(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
               const Fused &f = Fused());

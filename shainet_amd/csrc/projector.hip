@@ -298,7 +298,6 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
       flags_cap = want;
     }
     if (p.splits > 1 && !error_word()) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
-    if (++epoch == 0) epoch = 1;  // zero is what untouched flag words hold
     GemvArgs a = {};
     a.x = xin;
     a.x_stride = xs;
@@ -310,7 +309,6 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.y = y;
     a.partials = scratch.p;
     a.flags = flags;
-    a.epoch = epoch;
     a.error = error_word();
     a.T = T;
     a.K = K;
