@@ -58,11 +58,12 @@ struct DecodePlan {
 // wg_target: 0 = default
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
+size_t decode_flag_words(const DecodePlan &p);
 
 // q_rot: rotated queries [rows][H*hd]; the cache already holds the new rows.
 // before / after (here and in launch_prefill; nullable): events that receive the first clock
 // reading of the first kernel and the last one of the last kernel of the launch.
-// part_flag: DecodePlan::n_slots words of device memory, zero when allocated; the kernel
+// part_flag: decode_flag_words() words of device memory, zero when allocated; the kernel
 // leaves them zero.  error: an int the device can write (pinned host memory will do), set
 // to 1 when a workgroup gave up waiting for the partials of others.
 struct DecodeArgs {

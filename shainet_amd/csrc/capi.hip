@@ -183,7 +183,7 @@ Shape shape_of(const shainet_attn_ctx *c, int cap) {
   return sh;
 }
 
-// Zero-initialised words, one per partial slot of the decode split.
+// Zero-initialised flag words of the decode split.
 int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
   if (!error_word()) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
   if (n <= c->part_flag_cap) return SHAINET_HIP_OK;
@@ -220,7 +220,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
   if (path == Path::kDecodeSplitK) {
     const DecodePlan plan = plan_decode(st, sh, c->decode_wgs_override);
     int rc = c->partials.reserve(decode_partial_floats(sh, plan));
-    if (!rc) rc = ensure_decode_flags(c, (size_t)plan.n_slots, stream);
+    if (!rc) rc = ensure_decode_flags(c, decode_flag_words(plan), stream);
     if (rc) return rc;
     DecodeArgs d;
     d.q_rot = q_rot;

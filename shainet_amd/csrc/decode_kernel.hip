@@ -8,15 +8,16 @@
 // end in units of 16-key tiles and cut into equal contiguous spans, one per
 // workgroup, so every workgroup streams the same number of bytes whatever the
 // sequence lengths are.  A span that crosses a pair boundary is processed as two
-// segments.  The four wavefronts of a workgroup take the tiles of a segment
-// round-robin, each keeping its own online softmax, and merge through LDS into
-// one partial (max, sum, O) per segment; the workgroup that holds the end of a
-// pair waits, once its own span is done, for the partials of the workgroups that
-// hold the pair's earlier parts (a word per partial says when it is complete; the
-// merging workgroup clears it again),
-// merges them in a fixed order and writes the output row, so a decode step is one
-// launch.  Nothing a workgroup does between two segments waits for another
-// workgroup, and the next segment's first loads are in flight by then.
+// segments.  The four wavefronts of a workgroup take the tiles of the span
+// round-robin (across segments), each keeping its own online softmax per segment,
+// and merge through LDS into one partial (max, sum, O) per segment; the workgroup
+// that holds the end of a pair waits, once its own span is done, for the partials
+// of the workgroups that hold the pair's earlier parts (flag words say when a
+// partial is complete; the merging workgroup clears them again), merges them in a
+// fixed order and writes the output row, so a decode step is one launch.  Nothing
+// a workgroup does between two segments waits for another workgroup or for memory:
+// a wavefront's first tile of the next segment is fetched during its last tile of
+// this one, and a partial is marked complete one tile later.
 //
 // Per 16-key tile a wavefront
 //   * copies the K tile (16 contiguous rows) from HBM straight into LDS with
@@ -43,6 +44,7 @@
 
 #include <math.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace shainet {
 
@@ -59,6 +61,9 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // flag word written after them.
 __device__ __forceinline__ void coherent_store(float *p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coherent_store4(float *p, f32x4 v) {  // the same, 16 bytes at a time
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ float coherent_load(const float *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -129,8 +134,8 @@ __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const Se
 
 constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each
 
-// part_flag: one word per partial slot, zero between launches: a workgroup sets the word of a
-// partial it has completed, the workgroup that merges the pair clears the words it waited for
+// part_flag: NW words per partial slot, zero between launches: each wavefront sets its word of
+// a partial once its share is in memory, the workgroup that merges the pair clears the words it waited for
 // (so a launch may be replayed as it is).  error: set when the wait for other workgroups'
 // partials was given up.
 template <int HD, int NW>
@@ -141,13 +146,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
-  // rows [g][HD] in its second one while the first already receives the next segment's tile
+  // rows [g][HD] in one while the other already receives the next segment's first tile
   __shared__ __attribute__((aligned(1024))) char k_lds[NW][2][C::TILE_BYTES];
   __shared__ float sm_m[NW][16], sm_l[NW][16];  // per wavefront and head: running max, sum
+  __shared__ int sm_park[NW];                   // where each wavefront parked its O rows
   constexpr int TILE_FLOATS = C::TILE_BYTES / 4;
   constexpr int WAVE_LDS_FLOATS = 2 * TILE_FLOATS;  // floats between two wavefronts' areas
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile numbers stay in scalar registers
   const int col = lane & 15, j = lane >> 4;
   const int g = sh.g;
   const int t_begin = blockIdx.x * tiles_per_wg;
@@ -163,57 +170,89 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
 
   f32x4 v_next[4][C::NVU];
   float qr[HD / 4];
-  // first tile of a segment into the wavefront's first buffer, its V rows and the query rows
-  auto start_segment = [&](const Segment &sg) {
-    const int tile = sg.tile0 + wave;
-    if (tile < sg.tile1) {
-      issue_k_tile<HD>(sg.kbase, tile * 16, sg.L - 1, my_lds, lane);
-      load_v_tile<HD>(sg.vbase, tile * 16, sg.L - 1, col, j, v_next);
-    }
+  // columns beyond the group repeat head 0: their results are never stored, and leaving the
+  // loaded values untouched here keeps the wait for them out of this place
+  auto load_q = [&](const Segment &sg) {
     const float *qp = q_rot + ((long long)sg.token * sh.H + sg.kvh * g + (col < g ? col : 0)) * HD + 4 * j;
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      f32x4 x = *(const f32x4 *)(qp + 16 * i);
-      if (col >= g) x = f32x4{0.f, 0.f, 0.f, 0.f};
+      const f32x4 x = *(const f32x4 *)(qp + 16 * i);
       qr[4 * i + 0] = x.x;
       qr[4 * i + 1] = x.y;
       qr[4 * i + 2] = x.z;
       qr[4 * i + 3] = x.w;
     }
   };
-  start_segment(seg);
+  // `par`: the one of this wavefront's two buffers that holds (or is receiving) its next K tile.
+  // A segment's first tile is fetched while the segment before it is still being worked on.
+  int par = 0;
+  // The tiles of the span go to the wavefronts round-robin as one sequence, whatever segments
+  // they fall into (a fresh start per segment would leave one wavefront with a tile more than
+  // its share in every segment): the first tile of the segment at stream position ts for
+  // this wavefront.
+  auto first_tile = [&](const Segment &sg, int ts) { return sg.tile0 + ((wave - (ts - t_begin)) & (NW - 1)); };
+  static_assert((NW & (NW - 1)) == 0, "round-robin by masking");
+  // start fetching the tile at key row `row` into buffer `which`
+  auto fetch = [&](int which, const float *kb_, const float *vb_, int row, int last_row) {
+    issue_k_tile<HD>(kb_, row, last_row, my_lds + which * C::TILE_BYTES, lane);
+    load_v_tile<HD>(vb_, row, last_row, col, j, v_next);
+  };
+  if (first_tile(seg, t) < seg.tile1) fetch(0, seg.kbase, seg.vbase, first_tile(seg, t) * 16, seg.L - 1);
+  load_q(seg);
 
   // the pair whose last segment this workgroup holds without holding all of it: merged at the
   // end of the span (only a span's first segment can start inside a pair, so there is one at most)
   bool have_merge = false;
   Segment mseg = seg;
+  // this wavefront's share of a partial is written but not yet marked complete (slot, or -1):
+  // the mark follows the next wait for loads, which then also covers those stores
+  int pending = -1;
+  auto mark_pending = [&]() {
+    if (pending >= 0) {
+      if (lane == 0)
+        __hip_atomic_store(&part_flag[NW * pending + wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      pending = -1;
+    }
+  };
 
   for (;;) {
     const int L = seg.L, tile1 = seg.tile1;
     const float *kbase = seg.kbase, *vbase = seg.vbase;
+    // the segment after this one, if the span has one
+    const int t_next = t + (tile1 - seg.tile0);
+    const bool more = t_next < t_end;
+    Segment nseg = seg;
+    if (more) nseg = segment_at(t_next, t_end, s, st, sh, HD, kc, vc);
+    const int ntile = first_tile(nseg, t_next);
+    const bool nhave = more && ntile < nseg.tile1;
+
     float m = -INFINITY, l = 0.f;
     f32x4 o[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    int tile = seg.tile0 + wave;
-    for (int it = 0; tile < tile1; tile += NW, ++it) {
+    int tile = first_tile(seg, t);
+    // no tile of this segment for this wavefront: on to the next one's
+    if (tile >= tile1 && nhave) fetch(par, nseg.kbase, nseg.vbase, ntile * 16, nseg.L - 1);
+    for (; tile < tile1; tile += NW) {
       const int kb = tile * 16;
-      char *buf = my_lds + (it & 1) * C::TILE_BYTES;
+      const char *buf = my_lds + par * C::TILE_BYTES;
+      par ^= 1;
       // everything issued so far (this tile's K copy and V loads) has landed:
       // s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima), then a
       // compiler barrier so that no LDS read of the tile is scheduled above it
       __builtin_amdgcn_s_waitcnt(0x0F70);
       asm volatile("" ::: "memory");
+      mark_pending();
       f32x4 v_cur[4][C::NVU];
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
         for (int u = 0; u < C::NVU; ++u) v_cur[r][u] = v_next[r][u];
-      if (tile + NW < tile1) {
-        issue_k_tile<HD>(kbase, kb + 16 * NW, L - 1, my_lds + ((it + 1) & 1) * C::TILE_BYTES, lane);
-        load_v_tile<HD>(vbase, kb + 16 * NW, L - 1, col, j, v_next);
-      }
+      if (tile + NW < tile1)
+        fetch(par, kbase, vbase, kb + 16 * NW, L - 1);
+      else if (nhave)
+        fetch(par, nseg.kbase, nseg.vbase, ntile * 16, nseg.L - 1);
 
       f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
       const char *krow = buf + col * C::ROW_BYTES;
@@ -250,14 +289,16 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
           o[4 * u + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(v_cur[r][u].w, p[r], o[4 * u + 3], 0, 0, 0);
         }
     }
+    // the next segment's query rows (this one's are not needed any more)
+    if (more) load_q(nseg);
 
-    // merge the wavefronts through LDS: each one's tiles are consumed, so its second K tile
-    // buffer is free to hold its O rows
+    // merge the wavefronts through LDS: the wavefront parks its O rows [g][HD] in the one of
+    // its two buffers that does not hold (or receive) its next tile
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
-    float *sm_o = (float *)&k_lds[0][1][0];
+    float *sm_o = (float *)&k_lds[0][0][0];
     if (col < g) {
-      float *dst = sm_o + wave * WAVE_LDS_FLOATS + col * HD;
+      float *dst = sm_o + wave * WAVE_LDS_FLOATS + (par ^ 1) * TILE_FLOATS + col * HD;
 #pragma unroll
       for (int i = 0; i < NT; ++i)
 #pragma unroll
@@ -267,10 +308,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         sm_l[wave][col] = l;
       }
     }
+    if (lane == 0) sm_park[wave] = (par ^ 1) * TILE_FLOATS;
+    // a share of an earlier partial that is still unmarked (a wavefront that had no tile since)
+    if (pending >= 0) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      mark_pending();
+    }
     __syncthreads();
     const bool whole_pair = seg.tile0 == 0 && tile1 == seg.n_s;
     const int pair = seg.s * sh.KV + seg.kvh;
     const int slot = blockIdx.x + pair;  // unique: both terms only grow along the tile stream
+    int park[NW];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) park[w] = w * WAVE_LDS_FLOATS + sm_park[w];
     for (int idx = threadIdx.x; idx < g * HD; idx += 64 * NW) {
       const int cc = idx / HD, d = idx - cc * HD;
       float mm = sm_m[0][cc];
@@ -280,7 +330,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
         const float f = fast_exp2((sm_m[w][cc] - mm) * c);  // 0 for a wavefront that saw no tile
-        acc += f * sm_o[w * WAVE_LDS_FLOATS + cc * HD + d];
+        acc += f * sm_o[park[w] + cc * HD + d];
         ls += f * sm_l[w][cc];
       }
       if (whole_pair) {
@@ -299,24 +349,21 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       have_merge = true;
       mseg = seg;
     }
-    // The next segment's first loads go out before this one's partial is published: the wait
-    // below covers both.  (Its K tile lands in the wavefront's first buffer, which only this
-    // wavefront reads; the parked rows are in the second ones.)
-    t += tile1 - seg.tile0;
-    const bool more = t < t_end;
-    if (more) {
-      seg = segment_at(t, t_end, s, st, sh, HD, kc, vc);
-      start_segment(seg);
-    }
-    // Partials are written through to device-coherent memory (coherent_store); each wavefront
-    // waits for its stores to be acknowledged (s_waitcnt vmcnt(0): the barrier alone does not),
-    // then one lane marks the partial complete.  The barrier also ends the reads of the parked rows.
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    // Partials are written through to device-coherent memory (coherent_store).  Each
+    // wavefront marks its share complete in a word of its own once its stores are
+    // acknowledged, which the next wait for a tile tells (the barrier alone does not).
+    // The partial of a pair's end is read by this workgroup only.
+    if (!whole_pair && !pair_end && slot < n_slots) pending = slot;
+    // the parked rows are read: the next tiles may land there (with a copy into LDS in flight
+    // the barriers here also wait for this wavefront's loads: the compiler's rule, which is
+    // what a boundary inside a span still costs)
     __syncthreads();
-    if (!whole_pair && !pair_end && threadIdx.x == 0 && slot < n_slots)
-      __hip_atomic_store(&part_flag[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (!more) break;
+    seg = nseg;
+    t = t_next;
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // this wavefront's last stores are acknowledged
+  mark_pending();
 
   if (have_merge) {
     // This workgroup holds the end of a pair that others began: they have lower indices, were
@@ -326,13 +373,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const int n_part = (int)blockIdx.x - w_lo + 1;
     const int pair = mseg.s * sh.KV + mseg.kvh;
     if (wave == 0) {
-      unsigned *fl = part_flag + w_lo + pair;  // the last of the n_part partials is this workgroup's own
+      // NW words per partial; the last of the n_part partials is this workgroup's own
+      unsigned *fl = part_flag + NW * (w_lo + pair);
       for (int spins = 0;; ++spins) {
         bool ok = true;
-        for (int i = lane; i < n_part - 1; i += 64)
+        for (int i = lane; i < NW * (n_part - 1); i += 64)
           ok = ok && __hip_atomic_load(fl + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
         if (__all(ok)) {
-          for (int i = lane; i < n_part - 1; i += 64)
+          for (int i = lane; i < NW * (n_part - 1); i += 64)
             __hip_atomic_store(fl + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
@@ -417,6 +465,8 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
   return p;
 }
+
+size_t decode_flag_words(const DecodePlan &p) { return (size_t)p.n_slots * kDecodeWaves; }
 
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
   return (size_t)p.n_slots * sh.g * (sh.hd + 2);
