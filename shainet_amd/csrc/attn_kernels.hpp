@@ -52,6 +52,7 @@ int plan_work(SeqTable &st, const Shape &sh, Path path);
 struct DecodePlan {
   int total_tiles;
   int tiles_per_wg;
+  int skew;  // tiles an even workgroup takes more, and the odd one after it less, than tiles_per_wg
   int n_wgs;
   int n_slots;  // partial slots: workgroup index + pair index is unique per segment
 };

@@ -107,6 +107,17 @@ __device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last
   }
 }
 
+// Spans: workgroups 2k and 2k+1 share 2 * tiles_per_wg tiles of the stream, the even one taking
+// `skew` tiles more than half (workgroups go to the eight XCDs round-robin by index, and the
+// odd XCDs of the machines measured stream about 5 % slower than the even ones).
+__device__ __forceinline__ int span_begin(int w, int tiles_per_wg, int skew) {
+  return (w >> 1) * 2 * tiles_per_wg + ((w & 1) ? tiles_per_wg + skew : 0);
+}
+__device__ __forceinline__ int workgroup_of_tile(int t, int tiles_per_wg, int skew) {
+  const int k = t / (2 * tiles_per_wg);
+  return 2 * k + (t - k * 2 * tiles_per_wg >= tiles_per_wg + skew ? 1 : 0);
+}
+
 // One segment of a workgroup's span: tiles [tile0, tile1) of one (sequence, kv head) pair.
 struct Segment {
   int s, kvh, L, n_s, tile0, tile1, token;
@@ -142,7 +153,7 @@ template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, int *error,
-    SeqTable st, Shape sh, int tiles_per_wg, int total_tiles, int n_slots, float c) {
+    SeqTable st, Shape sh, int tiles_per_wg, int skew, int total_tiles, int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
@@ -157,8 +168,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile numbers stay in scalar registers
   const int col = lane & 15, j = lane >> 4;
   const int g = sh.g;
-  const int t_begin = blockIdx.x * tiles_per_wg;
-  const int t_end = min(total_tiles, t_begin + tiles_per_wg);
+  const int t_begin = span_begin(blockIdx.x, tiles_per_wg, skew);
+  const int t_end = min(total_tiles, span_begin(blockIdx.x + 1, tiles_per_wg, skew));
+  if (t_begin >= t_end) return;  // the skew can leave the last workgroup without tiles
   char *my_lds = &k_lds[wave][0][0];
 
   int t = t_begin;
@@ -369,7 +381,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     // This workgroup holds the end of a pair that others began: they have lower indices, were
     // started before this one and wait for nobody, so waiting for their partials is safe.
     const int a = st.work_off[mseg.s] + mseg.kvh * mseg.n_s;  // the pair's tiles are [a, a + n_s)
-    const int w_lo = a / tiles_per_wg;
+    const int w_lo = workgroup_of_tile(a, tiles_per_wg, skew);
     const int n_part = (int)blockIdx.x - w_lo + 1;
     const int pair = mseg.s * sh.KV + mseg.kvh;
     if (wave == 0) {
@@ -461,6 +473,11 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   int q = (p.total_tiles + wg_target - 1) / wg_target;
   if (q < kDecodeWaves) q = kDecodeWaves;
   p.tiles_per_wg = q;
+  // tiles moved from each odd workgroup to the even one before it (see span_begin), in
+  // thousandths of a span; not worth it for short spans
+  static const int skew_env = getenv("SHAINET_HIP_DECODE_SKEW") ? atoi(getenv("SHAINET_HIP_DECODE_SKEW")) : -1;
+  const int permille = skew_env >= 0 && skew_env <= 200 ? skew_env : 50;
+  p.skew = q >= 32 ? q * permille / 1000 : 0;
   p.n_wgs = (p.total_tiles + q - 1) / q;
   p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
   return p;
@@ -489,12 +506,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
     hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.skew,
                           p.total_tiles,
                           p.n_slots, c);
   else
     hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.skew,
                           p.total_tiles,
                           p.n_slots, c);
   hipError_t e = hipGetLastError();
