@@ -49,10 +49,14 @@ int plan_work(SeqTable &st, const Shape &sh, Path path);
 
 // Decode work split: the 16-key tiles of all (sequence, kv head) pairs laid end to
 // end (st.work_off = per-sequence prefix sums) and cut into equal spans.
+// Where the spans of eight consecutive workgroups begin within their 8 * tiles_per_wg tiles.
+struct SpanTable {
+  int off[9];
+};
 struct DecodePlan {
   int total_tiles;
   int tiles_per_wg;
-  int skew;  // tiles an even workgroup takes more, and the odd one after it less, than tiles_per_wg
+  SpanTable spans;
   int n_wgs;
   int n_slots;  // partial slots: workgroup index + pair index is unique per segment
 };

@@ -107,15 +107,19 @@ __device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last
   }
 }
 
-// Spans: workgroups 2k and 2k+1 share 2 * tiles_per_wg tiles of the stream, the even one taking
-// `skew` tiles more than half (workgroups go to the eight XCDs round-robin by index, and the
-// odd XCDs of the machines measured stream about 5 % slower than the even ones).
-__device__ __forceinline__ int span_begin(int w, int tiles_per_wg, int skew) {
-  return (w >> 1) * 2 * tiles_per_wg + ((w & 1) ? tiles_per_wg + skew : 0);
+// Spans: eight consecutive workgroups share 8 * tiles_per_wg tiles of the stream, workgroup
+// 8k + r taking tiles [off[r], off[r + 1]) of them (SpanTable, made by plan_decode).  Workgroups
+// go to the eight XCDs round-robin by index, and the XCDs of the machines measured do not
+// stream equally fast (see plan_decode), so equal spans would not end together.
+__device__ __forceinline__ int span_begin(int w, int tiles_per_wg, const SpanTable &sp) {
+  return (w >> 3) * 8 * tiles_per_wg + sp.off[w & 7];
 }
-__device__ __forceinline__ int workgroup_of_tile(int t, int tiles_per_wg, int skew) {
-  const int k = t / (2 * tiles_per_wg);
-  return 2 * k + (t - k * 2 * tiles_per_wg >= tiles_per_wg + skew ? 1 : 0);
+__device__ __forceinline__ int workgroup_of_tile(int t, int tiles_per_wg, const SpanTable &sp) {
+  const int k = t / (8 * tiles_per_wg), rel = t - k * 8 * tiles_per_wg;
+  int r = 0;
+#pragma unroll
+  for (int i = 1; i < 8; ++i) r += rel >= sp.off[i] ? 1 : 0;
+  return 8 * k + r;
 }
 
 // One segment of a workgroup's span: tiles [tile0, tile1) of one (sequence, kv head) pair.
@@ -153,7 +157,7 @@ template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, int *error,
-    SeqTable st, Shape sh, int tiles_per_wg, int skew, int total_tiles, int n_slots, float c) {
+    SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
@@ -168,9 +172,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile numbers stay in scalar registers
   const int col = lane & 15, j = lane >> 4;
   const int g = sh.g;
-  const int t_begin = span_begin(blockIdx.x, tiles_per_wg, skew);
-  const int t_end = min(total_tiles, span_begin(blockIdx.x + 1, tiles_per_wg, skew));
-  if (t_begin >= t_end) return;  // the skew can leave the last workgroup without tiles
+  const int t_begin = span_begin(blockIdx.x, tiles_per_wg, sp);
+  const int t_end = min(total_tiles, span_begin(blockIdx.x + 1, tiles_per_wg, sp));
+  if (t_begin >= t_end) return;  // unequal spans can leave the last workgroup without tiles
   char *my_lds = &k_lds[wave][0][0];
 
   int t = t_begin;
@@ -381,7 +385,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     // This workgroup holds the end of a pair that others began: they have lower indices, were
     // started before this one and wait for nobody, so waiting for their partials is safe.
     const int a = st.work_off[mseg.s] + mseg.kvh * mseg.n_s;  // the pair's tiles are [a, a + n_s)
-    const int w_lo = workgroup_of_tile(a, tiles_per_wg, skew);
+    const int w_lo = workgroup_of_tile(a, tiles_per_wg, sp);
     const int n_part = (int)blockIdx.x - w_lo + 1;
     const int pair = mseg.s * sh.KV + mseg.kvh;
     if (wave == 0) {
@@ -473,12 +477,38 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   int q = (p.total_tiles + wg_target - 1) / wg_target;
   if (q < kDecodeWaves) q = kDecodeWaves;
   p.tiles_per_wg = q;
-  // tiles moved from each odd workgroup to the even one before it (see span_begin), in
-  // thousandths of a span; not worth it for short spans
-  static const int skew_env = getenv("SHAINET_HIP_DECODE_SKEW") ? atoi(getenv("SHAINET_HIP_DECODE_SKEW")) : -1;
-  const int permille = skew_env >= 0 && skew_env <= 200 ? skew_env : 50;
-  p.skew = q >= 32 ? q * permille / 1000 : 0;
+  // Share of each of eight consecutive spans, in thousandths of an equal share, by the XCD the
+  // workgroup lands on (index mod 8).  With equal spans the workgroups on odd XCDs finished
+  // streaming about 5 % after those on even XCDs on every box traced (3 and 5 last, 0 and 6
+  // first; the finer pattern differs from box to box).  SHAINET_HIP_DECODE_SHARES: eight
+  // numbers, or "0" for equal spans.  Not worth it for short spans.
+  static const struct Shares {
+    int v[8] = {1050, 950, 1050, 950, 1050, 950, 1050, 950};
+    Shares() {
+      const char *env = getenv("SHAINET_HIP_DECODE_SHARES");
+      if (!env) return;
+      int w[8], n = 0;
+      for (const char *c = env; *c && n < 8;) {
+        char *end;
+        const long x = strtol(c, &end, 10);
+        if (end == c) break;
+        w[n++] = (int)x;
+        c = *end ? end + 1 : end;
+      }
+      for (int i = 0; i < 8; ++i) v[i] = n == 8 && w[i] >= 500 && w[i] <= 1500 ? w[i] : 1000;
+    }
+  } shares;
+  long long sum = 0, acc = 0;
+  for (int i = 0; i < 8; ++i) sum += shares.v[i];
+  for (int i = 0; i <= 8; ++i) {
+    p.spans.off[i] = q >= 32 ? (int)(acc * 8 * q / sum) : i * q;
+    if (i < 8) acc += shares.v[i];
+  }
+  // the first workgroup count whose spans cover the stream
   p.n_wgs = (p.total_tiles + q - 1) / q;
+  auto begin_of = [&](int w) { return (w >> 3) * 8 * q + p.spans.off[w & 7]; };
+  while (p.n_wgs > 1 && begin_of(p.n_wgs - 1) >= p.total_tiles) --p.n_wgs;
+  while (begin_of(p.n_wgs) < p.total_tiles) ++p.n_wgs;
   p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
   return p;
 }
@@ -506,12 +536,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
     hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.skew,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, c);
   else
     hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.skew,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, c);
   hipError_t e = hipGetLastError();
