@@ -356,6 +356,8 @@ def main():
         ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096], K),
         ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384], K),
         ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4, K),
+        # the headline shape with every sequence at the top of its length range (1.07 GB per step)
+        ("qwen3_8b_decode_b16_ctx8192", 32, 8, 128, 1e6, True, [8192 - K - W - 8] * 16, max(20, K // 2)),
     ]
     for name, H, KV, hd, th, norm, lens, k_ in decode_cfgs:
         if want(name):
