@@ -417,9 +417,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
     for (int cc = wave; cc < g; cc += NW) {
       const long long first = base + cc;
+      // the largest of the partials' maxima: from a pass of its own over them, or, when one
+      // round of loads covers all partials, from that round (one memory round trip less)
+      const bool one_round = n_part <= 8 * GROUPS;
       float mm = -INFINITY;
-      for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
-      for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
+      if (!one_round) {
+        for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
+        for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
+      }
       float ls = 0.f;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
       for (int i0 = 0; i0 < n_part; i0 += 8 * GROUPS) {  // eight rows in flight per lane
@@ -432,6 +437,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
           x[u] = *(const f32x4 *)&part_o[pi * HD + 4 * d4];
           f[u] = part_ml[2 * pi];
           lp[u] = part_ml[2 * pi + 1];
+        }
+        if (one_round) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (u * GROUPS + grp < n_part) mm = fmaxf(mm, f[u]);
+#pragma unroll
+          for (int o2 = LPR; o2 < 64; o2 <<= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));  // over the lanes of one d4
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
