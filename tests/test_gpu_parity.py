@@ -224,6 +224,32 @@ def test_decode_group_sizes(hip, g, hd):
         check_step(ctx, cache, blocks, r, [1])
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_decode_random_ragged_batches(hip, seed):
+    """Spans, segments and merges of the decode split over many shapes: a few to 64 sequences of
+    unrelated lengths (1 to 900 cached rows, so pairs of one tile next to pairs of fifty), every
+    group size, both head dims; twice per shape, the second call on the grown caches, and a
+    third on a shuffled subset."""
+    r0 = np.random.default_rng(1000 + seed)
+    hd = int(r0.choice([64, 128]))
+    KV = int(r0.choice([1, 2, 4, 8]))
+    g = int(r0.choice([1, 2, 4, 8]))
+    B = int(r0.choice([1, 2, 5, 16, 33, 64]))
+    top = int(r0.choice([20, 200, 900]))
+    lens = [int(x) for x in r0.integers(1, top + 1, B)]
+    ctx, cache, blocks, r = make_pair(hip, KV * g, KV, hd, 1e6, norm=bool(seed & 1), batch=B, capacity=top + 8,
+                                      seed=seed)
+    for s_, L in enumerate(lens):
+        kf, vf = (r.standard_normal((KV, L, hd)).astype(np.float32) for _ in range(2))
+        cache.fill(s_, kf, vf)
+        blocks[s_].fill_cache(kf, vf)
+    what = f"hd {hd} KV {KV} g {g} B {B} lens up to {top}"
+    for i in range(2):
+        assert check_step(ctx, cache, blocks, r, [1] * B, what=f"{what}, call {i}") < 1e-4
+    some = [int(x) for x in r0.permutation(B)[: max(1, B // 2)]]
+    check_step(ctx, cache, blocks, r, [1] * len(some), seq_ids=some, what=f"{what}, subset")
+
+
 def test_config3_qwen3_8b_batch16_varlen_decode(hip):
     import torch
 
