@@ -78,6 +78,10 @@ struct DecodeArgs {
   float *partials;
   unsigned *part_flag;
   int *error;
+  // for the test of the give-up path only: marks go to flag_set (decode_flag_words() words)
+  // instead of part_flag, and waiting ends after spin_limit polls; null / 0 otherwise
+  unsigned *flag_set;
+  int spin_limit;
 };
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr);

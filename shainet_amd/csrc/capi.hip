@@ -112,6 +112,7 @@ struct shainet_attn_ctx {
   // decode split: a word per partial slot that says when it is complete (zero between launches)
   unsigned *part_flag = nullptr;
   size_t part_flag_cap = 0;
+  bool test_lose_marks = false;  // SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS: exercises the give-up path
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
@@ -190,8 +191,9 @@ int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
   size_t want = c->part_flag_cap ? c->part_flag_cap : 1024;
   while (want < n) want *= 2;
   unsigned *np = nullptr;
-  HIP_TRY(hipMalloc((void **)&np, want * sizeof(unsigned)));
-  hipError_t e = hipMemsetAsync(np, 0, want * sizeof(unsigned), stream);
+  const size_t words = c->test_lose_marks ? 2 * want : want;  // second half: where lost marks go
+  HIP_TRY(hipMalloc((void **)&np, words * sizeof(unsigned)));
+  hipError_t e = hipMemsetAsync(np, 0, words * sizeof(unsigned), stream);
   if (e != hipSuccess) {
     (void)hipFree(np);
     return hip_fail(e, "hipMemsetAsync(partial flags)");
@@ -230,6 +232,8 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     d.partials = c->partials.p;
     d.part_flag = c->part_flag;
     d.error = error_word();
+    d.flag_set = c->test_lose_marks ? c->part_flag + c->part_flag_cap : nullptr;
+    d.spin_limit = c->test_lose_marks ? 2000 : 0;
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);
       if (e != hipSuccess) return hip_fail(e, "prep launch");
@@ -353,6 +357,7 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
     int v = atoi(env);
     if (v >= 1 && v <= 65536) c->decode_wgs_override = v;
   }
+  c->test_lose_marks = getenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS") != nullptr;
   if (const char *env = getenv("SHAINET_HIP_PREFILL_WGS_PER_CU")) c->prefill_wgs_per_cu = atoi(env);
   if (const char *env = getenv("SHAINET_HIP_PREFILL_SPLITS")) c->prefill_splits_override = atoi(env);
   int rc = SHAINET_HIP_OK;

@@ -147,17 +147,18 @@ __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const Se
   return g;
 }
 
-constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each
+constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each: seconds
 
 // part_flag: NW words per partial slot, zero between launches: each wavefront sets its word of
 // a partial once its share is in memory, the workgroup that merges the pair clears the words it waited for
 // (so a launch may be replayed as it is).  error: set when the wait for other workgroups'
-// partials was given up.
+// partials was given up, after spin_limit polls.  flag_set: where the marks are written; the
+// same as part_flag except in the test of that give-up, which sends them elsewhere.
 template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
-    float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, int *error,
-    SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, float c) {
+    float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
+    int spin_limit, int *error, SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   auto mark_pending = [&]() {
     if (pending >= 0) {
       if (lane == 0)
-        __hip_atomic_store(&part_flag[NW * pending + wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&flag_set[NW * pending + wave], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       pending = -1;
     }
   };
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
             __hip_atomic_store(fl + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
-        if (spins >= kFlagSpinLimit) {
+        if (spins >= spin_limit) {
           if (lane == 0) *error = 1;
           break;
         }
@@ -540,6 +541,8 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
     if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
       return hipErrorInvalidValue;
   if (!d.q_rot) return hipErrorInvalidValue;
+  unsigned *flag_set = d.flag_set ? d.flag_set : d.part_flag;
+  const int spin_limit = d.spin_limit > 0 ? d.spin_limit : kFlagSpinLimit;
   float *part_o = d.partials;
   float *part_ml = d.partials + (size_t)p.n_slots * sh.g * sh.hd;
   const float c = scale * kLog2e;
@@ -548,12 +551,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
     hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.spans,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, c);
   else
     hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, d.error, st, sh, p.tiles_per_wg, p.spans,
+                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, c);
   hipError_t e = hipGetLastError();

@@ -250,6 +250,28 @@ def test_decode_random_ragged_batches(hip, seed):
     check_step(ctx, cache, blocks, r, [1] * len(some), seq_ids=some, what=f"{what}, subset")
 
 
+def test_partials_that_never_arrive_are_reported(hip, monkeypatch):
+    """Failure handling of the decode split, forced from the host: with the test switch the
+    workgroups mark their partials complete in a place nobody looks at and the merging
+    workgroups stop polling after 2000 looks, so every kernel still ends by itself; the call
+    that waits for the stream must report it.  A context made without the switch is unaffected."""
+    import shainet_amd as sa
+
+    H, KV, hd = 8, 2, 64
+    monkeypatch.setenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS", "1")
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, capacity=3000, seed=3)
+    monkeypatch.delenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS")
+    kf, vf = (r.standard_normal((KV, 2500, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)  # 157 tiles per pair: every pair is spread over many workgroups
+    q, k, v = rows(r, 1, H, KV, hd)
+    with pytest.raises(sa.hip.HipError, match="gave up waiting"):
+        ctx.forward(cache, q, k, v, [1])
+    ctx2, cache2, blocks2, r2 = make_pair(hip, H, KV, hd, 1e6, capacity=3000, seed=3)
+    cache2.fill(0, kf, vf)
+    blocks2[0].fill_cache(kf, vf)
+    check_step(ctx2, cache2, blocks2, r2, [1])
+
+
 def test_config3_qwen3_8b_batch16_varlen_decode(hip):
     import torch
 
