@@ -513,9 +513,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 Path choose_path(const SeqTable &st, const Shape &sh) {
   if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
-  bool all_single = true;
-  for (int s = 0; s < st.n_seqs; ++s) all_single = all_single && st.n_new[s] == 1;
-  if (all_single && sh.g <= 16) return Path::kDecodeSplitK;
+  // a few new rows per sequence: rows x heads of a group fit the 16 columns of the split-K
+  // kernel's MFMA tiles, which then streams K and V once for all of them
+  bool few = true;
+  for (int s = 0; s < st.n_seqs; ++s) few = few && st.n_new[s] * sh.g <= 16;
+  if (few) return Path::kDecodeSplitK;
   return Path::kPrefillMfma;
 }
 

@@ -47,18 +47,20 @@ Path choose_path(const SeqTable &st, const Shape &sh);
 // Fills st.work_off for the prefill or generic path and returns the number of work items.
 int plan_work(SeqTable &st, const Shape &sh, Path path);
 
-// Decode work split: the 16-key tiles of all (sequence, kv head) pairs laid end to
-// end (st.work_off = per-sequence prefix sums) and cut into equal spans.
 // Where the spans of eight consecutive workgroups begin within their 8 * tiles_per_wg tiles.
 struct SpanTable {
   int off[9];
 };
+// Decode work split (a few new rows per sequence: rows x group size <= 16, the columns of one
+// MFMA tile): the 16-key tiles of all (sequence, kv head) pairs laid end to
+// end (st.work_off = per-sequence prefix sums) and cut into spans.
 struct DecodePlan {
   int total_tiles;
   int tiles_per_wg;
   SpanTable spans;
   int n_wgs;
   int n_slots;  // partial slots: workgroup index + pair index is unique per segment
+  int cols;     // columns (new rows x heads of a group) per partial: the most any sequence has, at most 16
 };
 // wg_target: 0 = default
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);

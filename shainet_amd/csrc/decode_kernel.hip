@@ -124,7 +124,7 @@ __device__ __forceinline__ int workgroup_of_tile(int t, int tiles_per_wg, const 
 
 // One segment of a workgroup's span: tiles [tile0, tile1) of one (sequence, kv head) pair.
 struct Segment {
-  int s, kvh, L, n_s, tile0, tile1, token;
+  int s, kvh, R, L, n_s, tile0, tile1, token;  // R new rows; L keys visible to the last of them
   const float *kbase, *vbase;
 };
 
@@ -134,7 +134,8 @@ __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const Se
   while (s + 1 < st.n_seqs && t >= st.work_off[s + 1]) ++s;
   Segment g;
   g.s = s;
-  g.L = st.start_pos[s] + 1;  // visible keys of the one new row
+  g.R = st.n_new[s];
+  g.L = st.start_pos[s] + g.R;  // visible keys of the last new row
   g.n_s = (g.L + 15) >> 4;    // tiles per kv head of this sequence
   const int rel = t - st.work_off[s];
   g.kvh = rel / g.n_s;
@@ -158,7 +159,8 @@ template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
-    int spin_limit, int *error, SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, float c) {
+    int spin_limit, int *error, SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, int pstride,
+    float c) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
@@ -187,10 +189,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
 
   f32x4 v_next[4][C::NVU];
   float qr[HD / 4];
-  // columns beyond the group repeat head 0: their results are never stored, and leaving the
+  // columns beyond the last repeat column 0: their results are never stored, and leaving the
   // loaded values untouched here keeps the wait for them out of this place
+  // MFMA column c of a segment is new row c / g, head c % g of the group (R * g <= 16 columns)
   auto load_q = [&](const Segment &sg) {
-    const float *qp = q_rot + ((long long)sg.token * sh.H + sg.kvh * g + (col < g ? col : 0)) * HD + 4 * j;
+    const int cq = col < sg.R * g ? col : 0, row = cq / g;
+    const float *qp = q_rot + ((long long)(sg.token + row) * sh.H + sg.kvh * g + (cq - row * g)) * HD + 4 * j;
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const f32x4 x = *(const f32x4 *)(qp + 16 * i);
@@ -235,6 +239,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   for (;;) {
     const int L = seg.L, tile1 = seg.tile1;
     const float *kbase = seg.kbase, *vbase = seg.vbase;
+    const int nc = seg.R * g;                                   // columns in use
+    const int Lc = L - (seg.R - 1 - (col < nc ? col : 0) / g);  // keys visible to this lane's column
     // the segment after this one, if the span has one
     const int t_next = t + (tile1 - seg.tile0);
     const bool more = t_next < t_end;
@@ -283,15 +289,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       }
       float sv[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sv[r] = (kb + 4 * j + r < L) ? s0[r] + s1[r] : -INFINITY;
+      for (int r = 0; r < 4; ++r) sv[r] = (kb + 4 * j + r < Lc) ? s0[r] + s1[r] : -INFINITY;
       float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float mnew = fmaxf(m, mx);  // finite: key kb is valid
-      const float alpha = fast_exp2((m - mnew) * c);
+      const float mnew = fmaxf(m, mx);
+      // with several new rows a column may not see any key of a late tile (-inf so far: 0 stands in)
+      const float mref = mnew == -INFINITY ? 0.f : mnew;
+      const float alpha = fast_exp2((m - mref) * c);
       float p[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) p[r] = fast_exp2((sv[r] - mnew) * c);
+      for (int r = 0; r < 4; ++r) p[r] = fast_exp2((sv[r] - mref) * c);
       l = l * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
       m = mnew;
 #pragma unroll
@@ -314,7 +322,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     float *sm_o = (float *)&k_lds[0][0][0];
-    if (col < g) {
+    if (col < nc) {
       float *dst = sm_o + wave * WAVE_LDS_FLOATS + (par ^ 1) * TILE_FLOATS + col * HD;
 #pragma unroll
       for (int i = 0; i < NT; ++i)
@@ -338,22 +346,24 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     int park[NW];
 #pragma unroll
     for (int w = 0; w < NW; ++w) park[w] = w * WAVE_LDS_FLOATS + sm_park[w];
-    for (int idx = threadIdx.x; idx < g * HD; idx += 64 * NW) {
+    for (int idx = threadIdx.x; idx < nc * HD; idx += 64 * NW) {
       const int cc = idx / HD, d = idx - cc * HD;
       float mm = sm_m[0][cc];
 #pragma unroll
       for (int w = 1; w < NW; ++w) mm = fmaxf(mm, sm_m[w][cc]);
+      const float mref = mm == -INFINITY ? 0.f : mm;  // no key of the segment visible to this column
       float acc = 0.f, ls = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
-        const float f = fast_exp2((sm_m[w][cc] - mm) * c);  // 0 for a wavefront that saw no tile
+        const float f = fast_exp2((sm_m[w][cc] - mref) * c);  // 0 for a wavefront that saw no visible key
         acc += f * sm_o[park[w] + cc * HD + d];
         ls += f * sm_l[w][cc];
       }
       if (whole_pair) {
-        out[((long long)seg.token * sh.H + seg.kvh * g + cc) * HD + d] = acc / ls;
+        const int row = cc / g;
+        out[((long long)(seg.token + row) * sh.H + seg.kvh * g + (cc - row * g)) * HD + d] = acc / ls;
       } else if (slot < n_slots) {
-        const long long pi = (long long)slot * g + cc;
+        const long long pi = (long long)slot * pstride + cc;
         coherent_store(&part_o[pi * HD + d], acc);
         if (d == 0) {
           coherent_store(&part_ml[2 * pi], mm);
@@ -415,15 +425,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     constexpr int LPR = HD / 4;       // lanes that cover one row with float4
     constexpr int GROUPS = 64 / LPR;  // partials handled side by side
     const int d4 = lane % LPR, grp = lane / LPR;
-    const long long base = (long long)(w_lo + pair) * g;  // partial of workgroup w, head cc: base + (w - w_lo)*g + cc
-    for (int cc = wave; cc < g; cc += NW) {
+    const long long base = (long long)(w_lo + pair) * pstride;  // partial of workgroup w, column cc: base + (w - w_lo) * pstride + cc
+    for (int cc = wave; cc < mseg.R * g; cc += NW) {
       const long long first = base + cc;
       // the largest of the partials' maxima: from a pass of its own over them, or, when one
       // round of loads covers all partials, from that round (one memory round trip less)
       const bool one_round = n_part <= 8 * GROUPS;
       float mm = -INFINITY;
       if (!one_round) {
-        for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * g)]);
+        for (int i = lane; i < n_part; i += 64) mm = fmaxf(mm, part_ml[2 * (first + (long long)i * pstride)]);
         for (int o2 = 32; o2 > 0; o2 >>= 1) mm = fmaxf(mm, __shfl_xor(mm, o2));
       }
       float ls = 0.f;
@@ -434,7 +444,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int i = i0 + u * GROUPS + grp;
-          const long long pi = first + (long long)min(i, n_part - 1) * g;
+          const long long pi = first + (long long)min(i, n_part - 1) * pstride;
           x[u] = *(const f32x4 *)&part_o[pi * HD + 4 * d4];
           f[u] = part_ml[2 * pi];
           lp[u] = part_ml[2 * pi + 1];
@@ -464,7 +474,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       }
       if (grp == 0) {
         const float inv = 1.0f / ls;
-        *(f32x4 *)&out[((long long)mseg.token * sh.H + mseg.kvh * g + cc) * HD + 4 * d4] = acc * inv;
+        const int row = cc / g;
+        *(f32x4 *)&out[((long long)(mseg.token + row) * sh.H + mseg.kvh * g + (cc - row * g)) * HD + 4 * d4] = acc * inv;
       }
     }
   }
@@ -479,7 +490,7 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   DecodePlan p;
   st.work_off[0] = 0;
   for (int s = 0; s < st.n_seqs; ++s)
-    st.work_off[s + 1] = st.work_off[s] + sh.KV * ((st.start_pos[s] + 1 + 15) / 16);
+    st.work_off[s + 1] = st.work_off[s] + sh.KV * ((st.start_pos[s] + st.n_new[s] + 15) / 16);
   p.total_tiles = st.work_off[st.n_seqs];
   // One workgroup on each of the 256 compute units.  Its four wavefronts keep 64 KiB
   // of K and V in flight, 16 MiB over the chip, which saturates HBM; twice as many
@@ -523,13 +534,15 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   while (p.n_wgs > 1 && begin_of(p.n_wgs - 1) >= p.total_tiles) --p.n_wgs;
   while (begin_of(p.n_wgs) < p.total_tiles) ++p.n_wgs;
   p.n_slots = p.n_wgs + st.n_seqs * sh.KV;
+  p.cols = 0;
+  for (int s = 0; s < st.n_seqs; ++s) p.cols = st.n_new[s] * sh.g > p.cols ? st.n_new[s] * sh.g : p.cols;
   return p;
 }
 
 size_t decode_flag_words(const DecodePlan &p) { return (size_t)p.n_slots * kDecodeWaves; }
 
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
-  return (size_t)p.n_slots * sh.g * (sh.hd + 2);
+  return (size_t)p.n_slots * p.cols * (sh.hd + 2);
 }
 
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
@@ -538,13 +551,14 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
       (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.part_flag || !d.error)
     return hipErrorInvalidValue;
   for (int s = 0; s < st.n_seqs; ++s)
-    if (st.n_new[s] != 1 || st.start_pos[s] < 0 || st.start_pos[s] + 1 > sh.cap || st.slot[s] < 0)
+    if (st.n_new[s] < 1 || st.n_new[s] * sh.g > 16 || st.n_new[s] * sh.g > p.cols || st.start_pos[s] < 0 ||
+        st.start_pos[s] + st.n_new[s] > sh.cap || st.slot[s] < 0)
       return hipErrorInvalidValue;
   if (!d.q_rot) return hipErrorInvalidValue;
   unsigned *flag_set = d.flag_set ? d.flag_set : d.part_flag;
   const int spin_limit = d.spin_limit > 0 ? d.spin_limit : kFlagSpinLimit;
   float *part_o = d.partials;
-  float *part_ml = d.partials + (size_t)p.n_slots * sh.g * sh.hd;
+  float *part_ml = d.partials + (size_t)p.n_slots * p.cols * sh.hd;
   const float c = scale * kLog2e;
   // before / after (nullable) receive the kernel's own first and last clock reading, not the
   // time at which the stream reached them: what is between two kernels stays out
@@ -553,12 +567,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
     hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
-                          p.n_slots, c);
+                          p.n_slots, p.cols, c);
   else
     hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
-                          p.n_slots, c);
+                          p.n_slots, p.cols, c);
   hipError_t e = hipGetLastError();
   return e;
 }

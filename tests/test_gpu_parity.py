@@ -250,6 +250,31 @@ def test_decode_random_ragged_batches(hip, seed):
     check_step(ctx, cache, blocks, r, [1] * len(some), seq_ids=some, what=f"{what}, subset")
 
 
+@pytest.mark.parametrize("KV,g,hd,B,rows_new,top", [
+    (8, 4, 128, 16, [4] * 16, 900),                 # rows x group = 16 columns, all in use
+    (8, 4, 128, 16, [1, 2, 3, 4] * 4, 900),         # every row count side by side
+    (2, 8, 64, 5, [2, 1, 2, 2, 1], 700),
+    (4, 1, 64, 3, [16, 9, 1], 400),                 # one head per group: up to 16 rows
+    (2, 16, 128, 2, [1, 1], 300),
+    (8, 4, 64, 4, [4, 4, 4, 4], 0),                 # from empty caches: later rows see more keys than earlier ones have
+    (8, 2, 128, 1, [7], 5000),
+])
+def test_few_new_rows_take_the_decode_split(hip, KV, g, hd, B, rows_new, top):
+    """A few new rows per sequence (rows x heads of a group <= 16) go through the split-K decode
+    kernel as further columns of its tiles: each row sees the keys up to its own position."""
+    r0 = np.random.default_rng(hd + B + top)
+    ctx, cache, blocks, r = make_pair(hip, KV * g, KV, hd, 1e6, norm=True, batch=B, capacity=top + 64, seed=top)
+    for s_ in range(B):
+        L = int(r0.integers(1, top + 1)) if top else 0
+        if L:
+            kf, vf = (r.standard_normal((KV, L, hd)).astype(np.float32) for _ in range(2))
+            cache.fill(s_, kf, vf)
+            blocks[s_].fill_cache(kf, vf)
+    for i in range(3):
+        assert check_step(ctx, cache, blocks, r, rows_new, what=f"call {i}") < 1e-4
+    check_cache_bits(cache, blocks)
+
+
 def test_partials_that_never_arrive_are_reported(hip, monkeypatch):
     """Failure handling of the decode split, forced from the host: with the test switch the
     workgroups mark their partials complete in a place nobody looks at and the merging
