@@ -22,6 +22,7 @@
 
 #include <math.h>
 #include <stdlib.h>
+#include <string.h>
 
 namespace shainet {
 
@@ -511,13 +512,34 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 }  // namespace
 
+bool decode_entries(const SeqTable &st, const Shape &sh, SeqTable &out) {
+  if (sh.g < 1 || sh.g > 16) return false;
+  const int per = 16 / sh.g;  // rows whose columns fill one tile
+  memset(&out, 0, sizeof out);
+  int n = 0;
+  for (int s = 0; s < st.n_seqs; ++s) {
+    const int groups = (st.n_new[s] + per - 1) / per;
+    if (groups > 2 || n + groups > kMaxSeqs) return false;
+    for (int k = 0; k < groups; ++k, ++n) {
+      const int first = k * per, rows = st.n_new[s] - first < per ? st.n_new[s] - first : per;
+      out.slot[n] = st.slot[s];
+      out.start_pos[n] = st.start_pos[s] + first;  // the rows before them are in the cache already
+      out.n_new[n] = rows;
+      out.tok_off[n] = st.tok_off[s] + first;
+    }
+  }
+  out.n_seqs = n;
+  out.tok_off[n] = st.tok_off[st.n_seqs];
+  return true;
+}
+
 Path choose_path(const SeqTable &st, const Shape &sh) {
   if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
   // a few new rows per sequence: rows x heads of a group fit the 16 columns of the split-K
-  // kernel's MFMA tiles, which then streams K and V once for all of them
-  bool few = true;
-  for (int s = 0; s < st.n_seqs; ++s) few = few && st.n_new[s] * sh.g <= 16;
-  if (few) return Path::kDecodeSplitK;
+  // kernel's MFMA tiles, which then streams K and V once for all of them; up to twice as many
+  // rows go to it as two entries (decode_entries), which still beats the key-chunked prefill
+  SeqTable tmp;
+  if (decode_entries(st, sh, tmp)) return Path::kDecodeSplitK;
   return Path::kPrefillMfma;
 }
 

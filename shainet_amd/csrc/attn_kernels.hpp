@@ -43,6 +43,11 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
 // Which attention kernel a call uses.
 enum class Path { kDecodeSplitK, kPrefillMfma, kGeneric };
 Path choose_path(const SeqTable &st, const Shape &sh);
+// The sequences as the split-K decode kernel takes them: one entry per sequence with up to
+// 16 / g new rows, two entries (the first 16 / g rows, then the rest, which see the first ones
+// as cached) with up to twice as many.  False when some sequence has more or the entries
+// do not fit a table.
+bool decode_entries(const SeqTable &st, const Shape &sh, SeqTable &out);
 
 // Fills st.work_off for the prefill or generic path and returns the number of work items.
 int plan_work(SeqTable &st, const Shape &sh, Path path);

@@ -220,7 +220,9 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     c->prof_events.push_back(ev1);
   }
   if (path == Path::kDecodeSplitK) {
-    const DecodePlan plan = plan_decode(st, sh, c->decode_wgs_override);
+    SeqTable att;  // the attention kernel's view: long runs of new rows as two entries
+    if (!decode_entries(st, sh, att)) return fail(SHAINET_HIP_ERR_RUNTIME, "decode entries do not fit");
+    const DecodePlan plan = plan_decode(att, sh, c->decode_wgs_override);
     int rc = c->partials.reserve(decode_partial_floats(sh, plan));
     if (!rc) rc = ensure_decode_flags(c, decode_flag_words(plan), stream);
     if (rc) return rc;
@@ -238,7 +240,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
       e = launch_prep(*prep, st, sh, total_tokens, stream);
       if (e != hipSuccess) return hip_fail(e, "prep launch");
     }
-    e = launch_decode(d, st, sh, plan, scale, stream, ev0, ev1);
+    e = launch_decode(d, att, sh, plan, scale, stream, ev0, ev1);
   } else {
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);

@@ -258,6 +258,9 @@ def test_decode_random_ragged_batches(hip, seed):
     (2, 16, 128, 2, [1, 1], 300),
     (8, 4, 64, 4, [4, 4, 4, 4], 0),                 # from empty caches: later rows see more keys than earlier ones have
     (8, 2, 128, 1, [7], 5000),
+    (8, 4, 128, 16, [8, 5, 7, 1] * 4, 900),         # more rows than one tile has columns: two entries each
+    (2, 8, 64, 3, [4, 3, 1], 600),
+    (4, 1, 64, 2, [32, 17], 300),
 ])
 def test_few_new_rows_take_the_decode_split(hip, KV, g, hd, B, rows_new, top):
     """A few new rows per sequence (rows x heads of a group <= 16) go through the split-K decode
