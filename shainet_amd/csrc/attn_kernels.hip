@@ -136,8 +136,10 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
     const float *qp = q_rot + qo_off + 4 * j;
 #pragma unroll
     for (int i = 0; i < NK4; ++i) {
-      f32x4 t = *(const f32x4 *)(qp + 8 * i);
-      if (!valid) t = f32x4{0.f, 0.f, 0.f, 0.f};
+      // (lanes past the last virtual row repeat the last row: their results are never used,
+      // and not touching the loaded values here lets the first K and V loads go out behind
+      // these instead of after their arrival)
+      const f32x4 t = *(const f32x4 *)(qp + 8 * i);
       qr[4 * i + 0] = t.x;
       qr[4 * i + 1] = t.y;
       qr[4 * i + 2] = t.z;
@@ -156,42 +158,37 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
   // group of wavefronts) travel global memory -> registers during one iteration and
   // registers -> LDS at the start of the next.
   f32x4 stage_k[LD4], stage_v[LD4];
-  auto load_k = [&](int sp) {
+  auto load_tiles = [&](f32x4 (&dst)[LD4], const float *base, int sp) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
       const int idx = threadIdx.x + NTHREADS * u;
       const int ts = idx / TILE4, rem = idx - ts * TILE4;
       const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
-      stage_k[u] = *(const f32x4 *)(kbase + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
+      dst[u] = *(const f32x4 *)(base + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
     }
   };
-  auto load_v = [&](int sp) {
+  auto park_k = [&](const f32x4 (&src)[LD4], int buf) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
       const int idx = threadIdx.x + NTHREADS * u;
       const int ts = idx / TILE4, rem = idx - ts * TILE4;
       const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
-      stage_v[u] = *(const f32x4 *)(vbase + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
+      *(f32x4 *)&Ks[buf][ts][r * KSTR + 4 * c4] = src[u];
     }
   };
-  auto store_k = [&](int buf) {
+  auto park_v = [&](const f32x4 (&src)[LD4], int buf) {
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
       const int idx = threadIdx.x + NTHREADS * u;
       const int ts = idx / TILE4, rem = idx - ts * TILE4;
       const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
-      *(f32x4 *)&Ks[buf][ts][r * KSTR + 4 * c4] = stage_k[u];
+      *(f32x4 *)&Vs[buf][ts][r * HD + 4 * c4] = src[u];
     }
   };
-  auto store_v = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + NTHREADS * u;
-      const int ts = idx / TILE4, rem = idx - ts * TILE4;
-      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
-      *(f32x4 *)&Vs[buf][ts][r * HD + 4 * c4] = stage_v[u];
-    }
-  };
+  auto load_k = [&](int sp) { load_tiles(stage_k, kbase, sp); };
+  auto load_v = [&](int sp) { load_tiles(stage_v, vbase, sp); };
+  auto store_k = [&](int buf) { park_k(stage_k, buf); };
+  auto store_v = [&](int buf) { park_v(stage_v, buf); };
 
   // S^T of one key tile: 32 keys x 32 virtual rows, K from LDS stage `buf`
   // MFMA operands come from LDS; every fetch is issued PF steps before the MFMAs
@@ -233,18 +230,22 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
 #pragma unroll
   for (int r = 0; r < 16; ++r) s_cur[r] = s_next[r] = 0.f;
   if (n_sp > 0) {
-    load_k(0);
-    load_v(0);
-    store_k(0);
-    store_v(0);
+    // everything the first step needs is requested at once, with registers of its own for
+    // the tiles that go to LDS right away: one memory round trip before the first MFMA
+    // instead of three
+    f32x4 k0[LD4], v0[LD4], k1[LD4];
+    load_tiles(k0, kbase, 0);
+    load_tiles(v0, vbase, 0);
     if (n_sp > 1) {
-      load_k(1);
+      load_tiles(k1, kbase, 1);
       load_v(1);
-      store_k(1);
     }
+    if (n_sp > 2) load_k(2);
+    park_k(k0, 0);
+    park_v(v0, 0);
+    if (n_sp > 1) park_k(k1, 1);
   }
   __syncthreads();
-  if (n_sp > 2) load_k(2);
   if (kt0 + gidx < kt1 && (kt0 + gidx) * 32 <= wave_hi) s_cur = scores(0);
   __syncthreads();  // step 0 overwrites Ks[0]
 
