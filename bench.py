@@ -370,6 +370,9 @@ def main():
         ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512, max(5, K // 10)),
         # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
         ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048, max(5, K // 10)),
+        # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
+        # through the split-K decode kernel as further columns of its tiles)
+        ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, lens3, 4, small),
     ]
     for name, H, KV, hd, th, norm, lens, T, k_ in prefill_cfgs:
         if want(name):
