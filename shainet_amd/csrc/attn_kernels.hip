@@ -18,8 +18,6 @@
 // pieces of K rows.
 #include "attn_kernels.hpp"
 
-#include <hip/hip_ext.h>
-
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -624,14 +622,15 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
     const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
     if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
   }
+  hipEvent_t main_after = ns == 1 ? after : nullptr;  // with key chunks the combine kernel ends the timed stretch
 #define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                    \
   do {                                                                                                          \
     if (groups == 2)                                                                                            \
-      hipExtLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, before,          \
-                            ns == 1 ? after : nullptr, 0, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);  \
+      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, before,           \
+                           main_after, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);                     \
     else                                                                                                        \
-      hipExtLaunchKernelGGL((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, before,          \
-                            ns == 1 ? after : nullptr, 0, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);  \
+      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, before,           \
+                           main_after, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);                     \
   } while (0)
   if (sh.hd == 64) {
     if (ns > 1)
@@ -647,8 +646,9 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
 #undef SHAINET_LAUNCH_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || ns == 1) return e;
-  hipExtLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, nullptr,
-                        after, 0, part_o, part_ml, out, st, sh, ns, c);
+  hipEvent_t none = nullptr;
+  SHAINET_LAUNCH_TIMED(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, none, after,
+                       part_o, part_ml, out, st, sh, ns, c);
   return hipGetLastError();
 }
 

@@ -2,6 +2,18 @@
 // launcher validates the shapes its kernel assumes and returns a hipError_t.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+// A kernel launch that hands the kernel's own first and last clock reading to two events when
+// there are any (hipExtLaunchKernel), and is a plain launch, as a caller's stream capture may
+// need it, when there are none.
+#define SHAINET_LAUNCH_TIMED(kernel, grid, block, lds, stream, before, after, ...)                         \
+  do {                                                                                                   \
+    if ((before) || (after))                                                                             \
+      hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, before, after, 0, __VA_ARGS__);            \
+    else                                                                                                 \
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                 \
+  } while (0)
 
 namespace shainet {
 

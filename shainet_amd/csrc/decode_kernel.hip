@@ -40,8 +40,6 @@
 //           key 4*j + r of the tile, where accumulator register r of S^T lives.
 #include "attn_kernels.hpp"
 
-#include <hip/hip_ext.h>
-
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -564,12 +562,12 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   // time at which the stream reached them: what is between two kernels stays out
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
   if (sh.hd == 64)
-    hipExtLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
+    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, p.cols, c);
   else
-    hipExtLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, 0, d.q_rot,
+    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
                           p.n_slots, p.cols, c);
