@@ -568,6 +568,33 @@ def test_device_pointer_mode_matches_host_pointer_mode(hip):
     assert np.array_equal(res[0], res[1])
 
 
+def test_two_contexts_decode_at_the_same_time(hip):
+    """Two contexts, each on its own stream, take decode calls in turn without waiting for each
+    other: their kernels share the chip, and each launch's merging workgroups wait only for
+    workgroups of their own launch."""
+    import torch
+
+    H, KV, hd, steps = 16, 4, 128, 12
+    sides = []
+    for seed, L in ((11, 3000), (12, 1700)):
+        ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, capacity=L + steps + 8, seed=seed)
+        kf, vf = (r.standard_normal((KV, L, hd)).astype(np.float32) for _ in range(2))
+        cache.fill(0, kf, vf)
+        blocks[0].fill_cache(kf, vf)
+        rows_ = [rows(r, 1, H, KV, hd) for _ in range(steps)]
+        dev = [[torch.from_numpy(a).cuda() for a in p] for p in rows_]
+        sides.append((ctx, cache, blocks[0], rows_, dev, []))
+    torch.cuda.synchronize()
+    for i in range(steps):
+        for ctx, cache, _, _, dev, outs in sides:
+            outs.append(ctx.forward(cache, *dev[i], [1]))  # device pointers: asynchronous
+    for ctx, cache, blk, rows_, _, outs in sides:
+        ctx.sync()
+        for i in range(steps):
+            want = blk.attention_cached_qkv(*rows_[i], threads=4)
+            rm.assert_close(outs[i].cpu().numpy(), want, ATOL, RTOL, f"step {i}")
+
+
 # ------------------------------------------------------------------ the layer, projections included
 def _layer_pair(hip, d, H, KV, hd, theta, seed, norm=False, bias=False, wscale=0.02):
     r = np.random.default_rng(seed)
