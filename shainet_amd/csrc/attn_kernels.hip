@@ -77,14 +77,13 @@ __device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &
 // second key tile, so that each SIMD holds two wavefronts of one workgroup and the
 // vector-ALU work of one hides behind the MFMAs of the other even when a launch
 // puts a single workgroup on a compute unit.  The two halves merge through LDS.
+// One workgroup's work: the row block (and key chunk) number `bid` of the launch.
 template <int HD, bool SPLIT, int G>
-__global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(const float *__restrict__ q_rot,
-                                                              const float *__restrict__ kc,
-                                                              const float *__restrict__ vc,
-                                                              float *__restrict__ out,
-                                                              float *__restrict__ part_o,
-                                                              float *__restrict__ part_ml, SeqTable st,
-                                                              Shape sh, int ns, float c) {
+__device__ __forceinline__ void prefill_block(const int bid, const float *__restrict__ q_rot,
+                                              const float *__restrict__ kc, const float *__restrict__ vc,
+                                              float *__restrict__ out, float *__restrict__ part_o,
+                                              float *__restrict__ part_ml, const SeqTable &st, const Shape &sh,
+                                              int ns, float c) {
   constexpr int NK4 = HD / 8;   // float4 pieces of a K row per lane
   constexpr int NT = HD / 32;   // d tiles of the output
   constexpr int KSTR = HD + 4;  // padded K row stride in LDS: conflict-free 16-byte reads down a column
@@ -100,9 +99,9 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
   // head and its K/V stay in that XCD's L2.  When a launch has too few row blocks to
   // fill the chip, each block's key range is cut into ns chunks that run as separate
   // workgroups and leave partial (max, sum, O) rows for prefill_combine_kernel.
-  const int kvh = blockIdx.x % sh.KV;
-  const int chunk = SPLIT ? (blockIdx.x / sh.KV) % ns : 0;
-  const int item = SPLIT ? blockIdx.x / sh.KV / ns : blockIdx.x / sh.KV;
+  const int kvh = bid % sh.KV;
+  const int chunk = SPLIT ? (bid / sh.KV) % ns : 0;
+  const int item = SPLIT ? bid / sh.KV / ns : bid / sh.KV;
   int s, vb;
   locate_block(st, item, s, vb);
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
@@ -396,6 +395,37 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
   }
 }
 
+template <int HD, bool SPLIT, int G>
+__global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(const float *__restrict__ q_rot,
+                                                              const float *__restrict__ kc,
+                                                              const float *__restrict__ vc,
+                                                              float *__restrict__ out,
+                                                              float *__restrict__ part_o,
+                                                              float *__restrict__ part_ml, SeqTable st,
+                                                              Shape sh, int ns, float c) {
+  prefill_block<HD, SPLIT, G>(blockIdx.x, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);
+}
+
+// For launches of two or three row blocks per compute unit: a workgroup takes, in turn, block b
+// of the launch (blocks are numbered by decreasing key range), block 2N - 1 - b and block
+// 2N + b (N workgroups): long, short and shorter ones that add up to about the same work for
+// every workgroup, instead of the dispatcher starting another workgroup where one has ended
+// (3.5 us later, measured).
+template <int HD, int G>
+__global__ __launch_bounds__(256 * G, 1) void prefill_turns_kernel(const float *__restrict__ q_rot,
+                                                                   const float *__restrict__ kc,
+                                                                   const float *__restrict__ vc,
+                                                                   float *__restrict__ out, SeqTable st, Shape sh,
+                                                                   int n_blocks, float c) {
+  const int N = gridDim.x, b = blockIdx.x;
+  for (int turn = 0; turn < 3; ++turn) {
+    const int bid = (turn & 1) ? (turn + 1) * N - 1 - b : turn * N + b;
+    if (bid >= n_blocks) continue;
+    if (turn) __syncthreads();  // the LDS stages are free: nobody is still merging the last block's halves
+    prefill_block<HD, false, G>(bid, q_rot, kc, vc, out, nullptr, nullptr, st, sh, 1, c);
+  }
+}
+
 // Merge the key chunks of one (row block, kv head): online-softmax combine per row.
 // Four workgroups per block (32 of its 128 virtual rows each, blockIdx.y) and up to eight
 // chunks' loads in flight per thread: the kernel is bound by load latency, not by bytes.
@@ -621,6 +651,20 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
     const size_t want = (size_t)160 * 1024 / wgs_per_cu;  // one more workgroup would not fit
     const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
     if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
+  }
+  static const bool turns_off = getenv("SHAINET_HIP_PREFILL_NO_TURNS") != nullptr;
+  // (only when the blocks fill those turns: otherwise compute units would stand idle where the
+  // dispatcher's own hand-out keeps them busy, 12 % slower at 640 blocks)
+  const int turns = (int)((n_wgs + 255) / 256);
+  if (!turns_off && ns == 1 && groups == 2 && n_wgs > 256 && n_wgs <= 768 && n_wgs * 100 >= (long long)turns * 256 * 97) {
+    dim3 fewer((unsigned)((n_wgs + turns - 1) / turns));
+    if (sh.hd == 64)
+      SHAINET_LAUNCH_TIMED((prefill_turns_kernel<64, 2>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, vc, out,
+                           st, sh, (int)n_wgs, c);
+    else
+      SHAINET_LAUNCH_TIMED((prefill_turns_kernel<128, 2>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, vc, out,
+                           st, sh, (int)n_wgs, c);
+    return hipGetLastError();
   }
   hipEvent_t main_after = ns == 1 ? after : nullptr;  // with key chunks the combine kernel ends the timed stretch
 #define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                    \
