@@ -417,11 +417,11 @@ def main():
     p = results.get("llama1b_prefill_t2048")
     if p:
         line["prefill_tflops"] = round(p["step_tflops"], 2)
-        line["roofline_prefill"] = {"bound": "mfma", "kernel": "prefill_mfma_kernel<64, false, 2>", "workload": p["workload"],
+        line["roofline_prefill"] = {"bound": "mfma", "kernel": "prefill_turns_kernel<64, 2>", "workload": p["workload"],
                                     "achieved": round(p["kernel_tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                                     "unit": "TFLOP/s", "frac": round(p["kernel_tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
                                     "kernel_us": round(p["kernel_us"], 2), "flops_per_launch": p["flops"],
-                                    "traffic": load_traffic("prefill_mfma_kernel<64, false, 2>", p["workload"])}
+                                    "traffic": load_traffic("prefill_turns_kernel<64, 2>", p["workload"])}
     print(json.dumps(line))
 
 
