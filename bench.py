@@ -275,6 +275,38 @@ def load_traffic(kernel, workload, bytes_per_launch=None):
     return t
 
 
+def yardsticks(torch, reps=5):
+    """What the device sustains on this box under the simplest possible load of each kind: a
+    plain coalesced read of 1 GiB (HBM) and a loop of nothing but fp32 MFMAs (matrix cores at
+    the clock the device holds under that load).  Reported next to the published peaks."""
+    from shainet_amd import hip
+
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 256 * 1024 * 1024
+    a = torch.empty(n, device="cuda").normal_()
+    sink = torch.zeros(256 * 512, device="cuda")
+    out = {}
+    flops = [0]
+
+    def mfma():
+        flops[0] = hip.mfma_f32_loop(sink, 4096, 256, stream)
+
+    for key, fn, amount in (("stream_read_gbps", lambda: hip.stream_read(a, sink, 768, stream), lambda: 4 * n / 1e3),
+                            ("mfma_f32_loop_tflops", mfma, lambda: flops[0] / 1e6)):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[key] = round(amount() / (e0.elapsed_time(e1) / reps * 1e3), 1)
+    del a
+    return out
+
+
 def calibrate(torch, sa, reps):
     """Plain copy and read kernels over 1 GiB: the bandwidth a perfectly coalesced stream
     reaches here, and (under rocprofv3 --pmc) what FETCH_SIZE / WRITE_SIZE read per byte."""
@@ -422,6 +454,8 @@ def main():
                                     "unit": "TFLOP/s", "frac": round(p["kernel_tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
                                     "kernel_us": round(p["kernel_us"], 2), "flops_per_launch": p["flops"],
                                     "traffic": load_traffic("prefill_turns_kernel<64, 2>", p["workload"])}
+    if not args.only:
+        line["yardsticks"] = yardsticks(torch)
     print(json.dumps(line))
 
 

@@ -334,6 +334,14 @@ int shainet_attn_profile_samples(shainet_attn_ctx *ctx, float *ms_out, int capac
 int shainet_hip_stream_copy_f32(const float *src, float *dst, long long n, int workgroups, void *stream);
 int shainet_hip_stream_read_f32(const float *src, float *sink, long long n, int workgroups, void *stream);
 
+/* A loop of nothing but fp32 MFMAs (v_mfma_f32_32x32x2_f32, four independent accumulators
+ * per wavefront): `workgroups` workgroups of 512 lanes run `iters` rounds of 16 MFMAs per
+ * wavefront and write one float per lane into sink[workgroups * 512]; *flops (nullable)
+ * receives the flops of the launch.  The rate it reaches is what the matrix cores sustain at
+ * the clock the device holds under that load, the yardstick next to the published peak for
+ * the prefill kernels.  No counterpart in the reference. */
+int shainet_hip_mfma_f32_loop(float *sink, int iters, int workgroups, long long *flops, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,7 +1,9 @@
 // Plain streaming kernels of known size.  They calibrate what the HBM counters of
 // rocprofv3 (FETCH_SIZE, WRITE_SIZE) read per byte moved and what bandwidth a
 // perfectly coalesced stream reaches on the device, the yardsticks the attention
-// kernels' traffic and bandwidth figures are compared with.
+// kernels' traffic and bandwidth figures are compared with.  A loop of nothing but
+// fp32 MFMAs does the same for the matrix cores: the rate they sustain at the clock
+// the device holds under that load, which the prefill kernels are compared with.
 #include <hip/hip_runtime.h>
 
 #include "../../include/shainet_hip_attn.h"
@@ -32,6 +34,32 @@ __global__ __launch_bounds__(256) void read_f32x4_kernel(const f32x4 *__restrict
   if ((threadIdx.x & 63) == 0) atomicAdd(&sink[blockIdx.x], s);
 }
 
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Every wavefront issues `iters` rounds of four independent v_mfma_f32_32x32x2_f32 (four
+// accumulators, so no instruction waits for the one before it) and folds the accumulators
+// into one float per lane so that the work cannot be dropped.
+__global__ __launch_bounds__(512, 1) void mfma_f32_loop_kernel(float *__restrict__ sink, int iters, float a0, float b0) {
+  f32x16 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  const float a = a0 + 1e-6f * threadIdx.x, b = b0;
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[t], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[t][r];
+  sink[(long long)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 }  // namespace
 
 extern "C" {
@@ -47,6 +75,15 @@ int shainet_hip_stream_read_f32(const float *src, float *sink, long long n, int 
   if (!src || !sink || n < 0 || (n & 3) || workgroups < 1) return SHAINET_HIP_ERR_ARGUMENT;
   hipLaunchKernelGGL(read_f32x4_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
                      (const f32x4 *)src, sink, n / 4);
+  return hipGetLastError() == hipSuccess ? SHAINET_HIP_OK : SHAINET_HIP_ERR_RUNTIME;
+}
+
+int shainet_hip_mfma_f32_loop(float *sink, int iters, int workgroups, long long *flops, void *stream) {
+  if (!sink || iters < 1 || workgroups < 1) return SHAINET_HIP_ERR_ARGUMENT;
+  hipLaunchKernelGGL(mfma_f32_loop_kernel, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream, sink, iters,
+                     0.5f, 0.25f);
+  // 16 MFMAs per round and wavefront, 2 * 32 * 32 * 2 flops each, 8 wavefronts per workgroup
+  if (flops) *flops = (long long)workgroups * 8 * iters * 16 * 4096;
   return hipGetLastError() == hipSuccess ? SHAINET_HIP_OK : SHAINET_HIP_ERR_RUNTIME;
 }
 

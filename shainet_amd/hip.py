@@ -126,6 +126,7 @@ _SIGNATURES = {
     "shainet_llama_model_topk": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), _f32p, C.POINTER(C.c_int)]),
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
+    "shainet_hip_mfma_f32_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_longlong), C.c_void_p]),
     "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
     "shainet_attn_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), _i32p]),
     "shainet_attn_profile_samples": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, _i32p]),
@@ -229,6 +230,13 @@ def stream_copy(src, dst, workgroups=4096, stream=None):
 def stream_read(src, sink, workgroups=4096, stream=None):
     """Plain read kernel; sink is a float tensor of at least `workgroups` elements."""
     _check(lib().shainet_hip_stream_read_f32(_ptr(src), _ptr(sink), src.numel(), workgroups, stream))
+
+
+def mfma_f32_loop(sink, iters, workgroups=256, stream=None):
+    """Loop of nothing but fp32 MFMAs; sink holds at least workgroups * 512 floats.  Returns the flops of the launch."""
+    flops = C.c_longlong(0)
+    _check(lib().shainet_hip_mfma_f32_loop(_ptr(sink), iters, workgroups, C.byref(flops), stream))
+    return flops.value
 
 
 class AttnContext:
