@@ -678,3 +678,41 @@ def test_c_abi_from_plain_c(hip):
                         "-lshainet_hip_kernels", "-lm", "-Wl,-rpath,$ORIGIN/../shainet_amd/lib"], check=True)
     done = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert done.returncode == 0 and "cabi_smoke ok" in done.stdout, done.stdout + done.stderr
+
+
+def test_yardstick_kernels_do_the_work_they_count(hip):
+    # the plain copy / read kernels and the MFMA loop that bench.py compares the attention kernels
+    # with: a yardstick that skipped part of its work would flatter every roofline fraction
+    import torch
+
+    from shainet_amd import hip as yard
+
+    n = 1 << 20
+    a = torch.arange(n, device="cuda", dtype=torch.float32) % 7.0
+    b = torch.zeros_like(a)
+    yard.stream_copy(a, b, 64)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    sink = torch.zeros(64, device="cuda")
+    yard.stream_read(a, sink, 64)
+    torch.cuda.synchronize()
+    assert float(sink.sum()) == float(a.double().sum())  # small integers: exact in any order
+
+    # every lane's 64 accumulator registers hold sum_k A[m][k] B[k][n] per MFMA with A[m][k] =
+    # 0.5 + 1e-6 * (32 k + m) and B = 0.25; a lane's registers cover 16 values of m (both lane halves
+    # together all 32), and each accumulator takes 4 MFMAs per round
+    iters, wgs = 3, 2
+    sink = torch.zeros(wgs * 512, device="cuda")
+    flops = yard.mfma_f32_loop(sink, iters, wgs)
+    torch.cuda.synchronize()
+    assert flops == wgs * 8 * iters * 16 * 2 * 32 * 32 * 2
+    got = sink.cpu().numpy().astype(np.float64).reshape(wgs, 8, 64)
+    lane_a = lambda wave, lane: 0.5 + 1e-6 * np.float32(64 * wave + lane).astype(np.float64)  # noqa: E731
+    for wave in range(8):
+        for lane in (0, 5, 31, 32, 63):
+            half = lane // 32
+            ms = [8 * (r // 4) + 4 * half + r % 4 for r in range(16)]
+            per_mfma = [0.25 * (lane_a(wave, m) + lane_a(wave, m + 32)) for m in ms]
+            want = 4 * (4 * iters) * sum(per_mfma)
+            assert abs(got[0, wave, lane] - want) < 1e-4 * want, (wave, lane, got[0, wave, lane], want)
+    assert np.array_equal(got[0], got[1])
