@@ -144,7 +144,22 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     }
   }
 
-  float m = -INFINITY, l = 0.f;
+  // Online softmax against a reference value per virtual row instead of the running maximum.
+  // The fp32 MFMAs run on the lanes of the vector ALU (a wavefront's vector instructions and
+  // MFMAs, its own or its SIMD neighbour's, never overlap: measured, 6 cycles per fma and 12
+  // per exp2 added to a stream of 64-cycle MFMAs), so every vector instruction of the tile loop
+  // is paid in matrix throughput.  Hence:
+  //   * the query rows are scaled by scale * log2(e) once, so scores come out in log2 units;
+  //   * the score accumulator starts at -m_ref instead of 0, so the MFMAs deliver s - m_ref;
+  //   * m_ref is only moved (and l, O rescaled) when a score exceeds it by more than kTau, or
+  //     for a row's first visible key; probabilities are then at most 2^kTau, no overflow.
+  // A tile on the common path costs a maximum, 16 exp2 and 16 adds per lane.
+  constexpr float kTau = 8.f;
+  float m_ref = 0.f, l = 0.f;
+  float thr = -INFINITY;  // a row's scores move m_ref when above this: anything finite until its first key, kTau after
+  f32x16 neg_m;           // -m_ref in all registers: the score MFMAs' initial accumulator
+#pragma unroll
+  for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
   f32x16 o[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -192,9 +207,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   // that use it, so that the matrix pipe never waits for an LDS round trip.
   auto scores = [&](int buf) {
     constexpr int PF = 2;
-    f32x16 sacc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    f32x16 sacc = neg_m;
     const float *kl = &Ks[buf][gidx][n * KSTR + 4 * j];
     f32x4 kv[NK4];
 #pragma unroll
@@ -242,6 +255,8 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     park_v(v0, 0);
     if (n_sp > 1) park_k(k1, 1);
   }
+#pragma unroll
+  for (int i = 0; i < HD / 2; ++i) qr[i] *= c;
   __syncthreads();
   if (kt0 + gidx < kt1 && (kt0 + gidx) * 32 <= wave_hi) s_cur = scores(0);
   __syncthreads();  // step 0 overwrites Ks[0]
@@ -264,82 +279,79 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     }
   };
 
-  // tiles [0, n_interior) are visible to every row of this wavefront: no masking
-  const int n_interior = wave_active ? (wave_lo + 1) / 32 : 0;
-
-  for (int sp = 0; sp < n_sp; ++sp) {
+  // One step; `cur` holds this step's scores, `nxt` receives the next step's.  For head_dim 64
+  // the loop below calls it with the two register sets swapping roles, so that nothing is
+  // copied between steps (T = 2048: 161 -> 154 us).
+  auto step = [&](const int sp, f32x16 &cur, f32x16 &nxt) {
     const int buf = sp & 1;
     const int kt = kt0 + G * sp + gidx, kt_next = kt + G;  // this group's tile now and in the next step
     if (sp + 2 < n_sp) store_k(buf);
     if (sp + 1 < n_sp) store_v(buf ^ 1);
     if (sp + 3 < n_sp) load_k(sp + 3);
     if (sp + 2 < n_sp) load_v(sp + 2);
-    if (kt_next < n_interior && kt_next < kt1) {
-      // Hot path, one basic block: the score MFMAs of tile kt+1 and the softmax
-      // arithmetic of tile kt are independent, so the scheduler can interleave them.
-      s_next = scores(buf ^ 1);
-      f32x16 sacc = s_cur;
-      float mx = sacc[0];
-#pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float mnew = fmaxf(m, mx);  // finite: the tile is fully visible
-      const float alpha = fast_exp2((m - mnew) * c);
-      const float mc = mnew * c;
-      float psum = 0.f;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sacc[r] = fast_exp2(sacc[r] * c - mc);
-        psum += sacc[r];
-      }
-      l = l * alpha + psum;
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-      m = mnew;
-      accumulate(sacc, buf);
-    } else {
-      if (kt_next < kt1 && kt_next * 32 <= wave_hi) s_next = scores(buf ^ 1);
-      if (kt < kt1 && kt * 32 <= wave_hi) {
-        f32x16 sacc = s_cur;
-        if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = kt * 32 + 8 * (r >> 2) + 4 * j + (r & 3);
-            if (key > lim) sacc[r] = -INFINITY;
-          }
-        }
-        float mx = sacc[0];
-#pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, sacc[r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float mnew = fmaxf(m, mx);
-        // a key chunk (or, with two groups, the second group's first tile) that starts past
-        // a row's last visible key leaves that row at -inf
-        const float mref = (SPLIT || G == 2) && mnew == -INFINITY ? 0.f : mnew;
-        const float alpha = fast_exp2((m - mref) * c);
-        const float mc = mref * c;
-        float psum = 0.f;
+    const bool have_next = kt_next < kt1 && kt_next * 32 <= wave_hi;
+    const bool have_cur = kt < kt1 && kt * 32 <= wave_hi;
+    if (have_next) nxt = scores(buf ^ 1);
+    if (have_cur) {
+      f32x16 sacc = cur;             // scores of tile kt minus m_ref, log2 units
+      if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          sacc[r] = fast_exp2(sacc[r] * c - mc);
-          psum += sacc[r];
+          const int key = kt * 32 + 8 * (r >> 2) + 4 * j + (r & 3);
+          if (key > lim) sacc[r] = -INFINITY;
         }
-        l = l * alpha + psum;
+      }
+      float mx = fmaxf(fmaxf(sacc[0], sacc[1]), sacc[2]);
+#pragma unroll
+      for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, sacc[r]), sacc[r + 1]);
+      mx = fmaxf(mx, sacc[15]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const bool move = mx > thr;  // never for a row without a visible key in this tile (mx = -inf)
+      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        // rare after a row's first tiles: move the reference to this tile's maximum
+        const float delta = move ? mx : 0.f;
+        const float alpha = (move && thr != -INFINITY) ? fast_exp2(-delta) : 1.f;  // nothing to rescale before a row's first key
+        m_ref += delta;
+        l *= alpha;
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[t][r] *= alpha;
-        m = mnew;
-        accumulate(sacc, buf);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sacc[r] -= delta;
+          nxt[r] -= delta;     // computed against the old reference (unused if there is no next tile)
+          neg_m[r] = -m_ref;
+        }
+        if (move) thr = kTau;
       }
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sacc[r] = fast_exp2(sacc[r]);
+        psum += sacc[r];
+      }
+      l += psum;
+      accumulate(sacc, buf);
     }
-    s_cur = s_next;
     __syncthreads();
+  };
+  if constexpr (HD == 64) {
+    for (int sp = 0; sp < n_sp; sp += 2) {
+      step(sp, s_cur, s_next);
+      if (sp + 1 < n_sp) step(sp + 1, s_next, s_cur);
+    }
+  } else {  // head_dim 128 has no registers left for the second copy of the step (it spills: measured slower)
+    for (int sp = 0; sp < n_sp; ++sp) {
+      step(sp, s_cur, s_next);
+      s_cur = s_next;
+    }
   }
 
   l += __shfl_xor(l, 32);
+  // what the merges below call the maximum: the reference the sums are relative to, in log2
+  // units, or -inf for a row that saw no key (its l and O are 0)
+  float m = thr == -INFINITY ? -INFINITY : m_ref;
   if constexpr (G == 2) {
     // the second group hands its (max, sum, O) to the first through the tile stages
     // (every wavefront is past the last step's barrier: nobody reads tiles any more)
@@ -358,8 +370,8 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     const float m1 = xm[wave * 64 + lane], l1 = xm[256 + wave * 64 + lane];
     const float mnew = fmaxf(m, m1);
     // a side that saw no visible key has max -inf: its factor is 0 (and both may be, in a key chunk)
-    const float a0 = m == -INFINITY ? 0.f : fast_exp2((m - mnew) * c);
-    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2((m1 - mnew) * c);
+    const float a0 = m == -INFINITY ? 0.f : fast_exp2(m - mnew);
+    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - mnew);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -692,7 +704,7 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
   if (e != hipSuccess || ns == 1) return e;
   hipEvent_t none = nullptr;
   SHAINET_LAUNCH_TIMED(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, none, after,
-                       part_o, part_ml, out, st, sh, ns, c);
+                       part_o, part_ml, out, st, sh, ns, 1.0f);  // the partials' maxima are already in log2 units
   return hipGetLastError();
 }
 
