@@ -305,10 +305,13 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
 #pragma unroll
       for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, sacc[r]), sacc[r + 1]);
       mx = fmaxf(mx, sacc[15]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const bool move = mx > thr;  // never for a row without a visible key in this tile (mx = -inf)
-      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      // mx covers this lane's half of the row's keys in the tile; the row's maximum is above thr
+      // exactly when one of the two halves' is (never for a row without a visible key here:
+      // -inf), so the halves only exchange their maxima once a move is certain
+      if (__builtin_amdgcn_ballot_w64(mx > thr) != 0) {
         // rare after a row's first tiles: move the reference to this tile's maximum
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const bool move = mx > thr;
         const float delta = move ? mx : 0.f;
         const float alpha = (move && thr != -INFINITY) ? fast_exp2(-delta) : 1.f;  // nothing to rescale before a row's first key
         m_ref += delta;
