@@ -104,11 +104,17 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   const int item = SPLIT ? bid / sh.KV / ns : bid / sh.KV;
   int s, vb;
   locate_block(st, item, s, vb);
+  // These are the same for all lanes of a wavefront, which the compiler cannot see: said so,
+  // tile counts, loop conditions and address bases live in scalar registers and their
+  // arithmetic leaves the vector ALU, which the MFMAs need
+  auto uniform = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+  s = uniform(s);
+  vb = uniform(vb);
   const int g = sh.g, T = st.n_new[s], S = st.start_pos[s];
   const int L = S + T, VR = T * g;
   const int lane = threadIdx.x & 63;
-  const int wave = (threadIdx.x >> 6) & 3;  // which 32 virtual rows of the block
-  const int gidx = threadIdx.x >> 8;        // which share of the key tiles (always 0 for G = 1)
+  const int wave = uniform((threadIdx.x >> 6) & 3);  // which 32 virtual rows of the block
+  const int gidx = uniform(threadIdx.x >> 8);        // which share of the key tiles (always 0 for G = 1)
   const int n = lane & 31, j = lane >> 5;
   const int v0 = vb * 128 + wave * 32;
   const bool wave_active = v0 < VR;
