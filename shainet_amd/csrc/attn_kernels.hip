@@ -176,13 +176,25 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   // group of wavefronts) travel global memory -> registers during one iteration and
   // registers -> LDS at the start of the next.
   f32x4 stage_k[LD4], stage_v[LD4];
+  // what a thread fetches of a step's G tiles does not change from step to step: row
+  // row_in_step[u] of the step's 32 G rows, columns col4 .. col4 + 3
+  int row_in_step[LD4];
+#pragma unroll
+  for (int u = 0; u < LD4; ++u) {
+    const int idx = threadIdx.x + NTHREADS * u;
+    const int ts = idx / TILE4, rem = idx - ts * TILE4;
+    row_in_step[u] = ts * 32 + rem / (HD / 4);
+  }
+  const unsigned col_bytes = 16u * (threadIdx.x % (HD / 4));  // NTHREADS is a multiple of HD / 4
+  static_assert(NTHREADS % (HD / 4) == 0, "a thread keeps its columns");
+  // a scalar base and a 32-bit byte offset per lane (a head's rows span less than 4 GiB: checked
+  // at launch); rows past the last one repeat it
   auto load_tiles = [&](f32x4 (&dst)[LD4], const float *base, int sp) {
+    const int first_row = (kt0 + G * sp) * 32;
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const int idx = threadIdx.x + NTHREADS * u;
-      const int ts = idx / TILE4, rem = idx - ts * TILE4;
-      const int r = rem / (HD / 4), c4 = rem - r * (HD / 4);
-      dst[u] = *(const f32x4 *)(base + (long long)min((kt0 + G * sp + ts) * 32 + r, L - 1) * HD + 4 * c4);
+      const unsigned off = (unsigned)min(first_row + row_in_step[u], L - 1) * (unsigned)(HD * 4) + col_bytes;
+      dst[u] = *(const f32x4 *)((const char *)base + off);
     }
   };
   auto park_k = [&](const f32x4 (&src)[LD4], int buf) {
@@ -299,7 +311,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     const bool have_cur = kt < kt1 && kt * 32 <= wave_hi;
     if (have_next) nxt = scores(buf ^ 1);
     if (have_cur) {
-      f32x16 sacc = cur;             // scores of tile kt minus m_ref, log2 units
+      f32x16 &sacc = cur;            // scores of tile kt minus m_ref, log2 units; not needed after this step
       if (kt * 32 + 31 > wave_lo) {  // tile crosses the diagonal for some row of this wavefront
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -652,6 +664,8 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
     return hipErrorInvalidValue;
   const long long n_wgs = (long long)items * sh.KV * ns;
   if (n_wgs > 0x7fffffffLL) return hipErrorInvalidValue;
+  // the kernels address a row of a (sequence, kv head) by a 32-bit byte offset from its first row
+  if ((long long)sh.cap * sh.hd * 4 > 0xffffffffLL) return hipErrorInvalidValue;
   const float c = scale * kLog2e;
   dim3 grid((unsigned)n_wgs);
   float *part_o = partials;
