@@ -716,3 +716,40 @@ def test_yardstick_kernels_do_the_work_they_count(hip):
             want = 4 * (4 * iters) * sum(per_mfma)
             assert abs(got[0, wave, lane] - want) < 1e-4 * want, (wave, lane, got[0, wave, lane], want)
     assert np.array_equal(got[0], got[1])
+
+
+@pytest.mark.parametrize("splits", [0, 3])
+@pytest.mark.parametrize("H,KV,hd", [(8, 2, 64), (4, 1, 128)])
+def test_prefill_scores_far_from_unit_scale(hip, H, KV, hd, splits, monkeypatch):
+    # The MFMA prefill kernels keep a reference value per row that moves only when a score exceeds it
+    # by 2^8, and take scores relative to it straight from the accumulator: score sequences that climb
+    # or fall by more than that from tile to tile, jump between +-hundreds, or have a huge spread must
+    # come out as the oracle's running-maximum softmax does.  Scores are steered through the last
+    # rotation pair, which RoPE (theta 1e6) turns by less than 1e-3 rad over these positions.
+    if splits:
+        monkeypatch.setenv("SHAINET_HIP_PREFILL_SPLITS", str(splits))
+    S, T = 70, 200
+    L = S + T
+    pos = np.arange(L, dtype=np.float64)
+    shapes = {
+        "climbing": 3.0 * pos,                                 # every tile's maximum is 96 above the last one's
+        "falling": -3.0 * pos,                                 # the first key dominates; later ones underflow
+        "sawtooth": 400.0 * ((pos // 32) % 2) - 200.0,         # whole tiles at -200 and +200 in turn
+        "late_spike": np.where(pos == L - 40, 500.0, -500.0),  # one key 1000 above all others
+    }
+    r = np.random.default_rng(hd + splits)
+    for name, target in shapes.items():
+        ctx, cache, blocks, _ = make_pair(hip, H, KV, hd, 1e6, capacity=512, seed=3)
+        d = hd - 1                                   # second half of the last rotation pair
+        k = np.zeros((L, KV * hd), np.float32)
+        q = np.zeros((L, H * hd), np.float32)
+        v = r.standard_normal((L, KV * hd)).astype(np.float32)
+        k[:, d::hd] = (target / 16.0)[:, None]
+        q[:, d::hd] = 16.0 * np.sqrt(hd)             # score = q k / sqrt(hd) = target
+        q += 0.01 * r.standard_normal(q.shape).astype(np.float32)
+        k += 0.01 * r.standard_normal(k.shape).astype(np.float32)
+        for lo, hi in ((0, S), (S, L)):
+            got = ctx.forward(cache, q[lo:hi], k[lo:hi], v[lo:hi], [hi - lo])
+            want = blocks[0].attention_cached_qkv(q[lo:hi], k[lo:hi], v[lo:hi], threads=8)
+            assert np.isfinite(got).all(), name
+            rm.assert_close(got, want, ATOL, RTOL, f"{name} hd={hd} rows {lo}..{hi}")
