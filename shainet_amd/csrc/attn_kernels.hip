@@ -163,9 +163,14 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   constexpr float kTau = 8.f;
   float m_ref = 0.f, l = 0.f;
   float thr = -INFINITY;  // a row's scores move m_ref when above this: anything finite until its first key, kTau after
-  f32x16 neg_m;           // -m_ref in all registers: the score MFMAs' initial accumulator
+  // -m_ref as the score MFMAs' initial accumulator: sixteen registers that hold it, or, where
+  // registers are short (head_dim 128), one more MFMA per tile that multiplies it by a column
+  // of ones
+  constexpr bool kRefByMfma = HD == 128;
+  f32x16 neg_m;
 #pragma unroll
   for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
+  const float ones_col = j == 0 ? 1.f : 0.f;  // A[key][k]: 1 for k = 0
   f32x16 o[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -225,7 +230,14 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   // that use it, so that the matrix pipe never waits for an LDS round trip.
   auto scores = [&](int buf) {
     constexpr int PF = 2;
-    f32x16 sacc = neg_m;
+    f32x16 sacc;
+    if constexpr (kRefByMfma) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+      sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ones_col, -m_ref, sacc, 0, 0, 0);
+    } else {
+      sacc = neg_m;
+    }
     const float *kl = &Ks[buf][gidx][n * KSTR + 4 * j];
     f32x4 kv[NK4];
 #pragma unroll
@@ -297,9 +309,9 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     }
   };
 
-  // One step; `cur` holds this step's scores, `nxt` receives the next step's.  For head_dim 64
-  // the loop below calls it with the two register sets swapping roles, so that nothing is
-  // copied between steps (T = 2048: 161 -> 154 us).
+  // One step; `cur` holds this step's scores, `nxt` receives the next step's.  The loop below
+  // calls it with the two register sets swapping roles, so that nothing is copied between
+  // steps (T = 2048: 161 -> 154 us).
   auto step = [&](const int sp, f32x16 &cur, f32x16 &nxt) {
     const int buf = sp & 1;
     const int kt = kt0 + G * sp + gidx, kt_next = kt + G;  // this group's tile now and in the next step
@@ -342,7 +354,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
         for (int r = 0; r < 16; ++r) {
           sacc[r] -= delta;
           nxt[r] -= delta;     // computed against the old reference (unused if there is no next tile)
-          neg_m[r] = -m_ref;
+          if constexpr (!kRefByMfma) neg_m[r] = -m_ref;
         }
         if (move) thr = kTau;
       }
@@ -357,16 +369,9 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     }
     __syncthreads();
   };
-  if constexpr (HD == 64) {
-    for (int sp = 0; sp < n_sp; sp += 2) {
-      step(sp, s_cur, s_next);
-      if (sp + 1 < n_sp) step(sp + 1, s_next, s_cur);
-    }
-  } else {  // head_dim 128 has no registers left for the second copy of the step (it spills: measured slower)
-    for (int sp = 0; sp < n_sp; ++sp) {
-      step(sp, s_cur, s_next);
-      s_cur = s_next;
-    }
+  for (int sp = 0; sp < n_sp; sp += 2) {
+    step(sp, s_cur, s_next);
+    if (sp + 1 < n_sp) step(sp + 1, s_next, s_cur);
   }
 
   l += __shfl_xor(l, 32);
