@@ -193,6 +193,38 @@ def cpu_baseline(w, reps):
     return times[len(times) // 2] * 1e6
 
 
+def cpu_baseline_prefill(reps=3):
+    """The oracle, one thread, on a bounded part of the 2048-row causal prefill of the Llama-3.2-1B
+    shape: its last 64 rows on top of the 1984 rows before them, extrapolated to the whole prefill
+    by the multiply-adds of the head loop (the scalar path's time is proportional to them)."""
+    import numpy as np
+
+    from oracle import oracle as orc
+
+    H, KV, hd, T, n_rows = 32, 8, 64, 2048, 64
+    r = np.random.default_rng(4)
+    b = orc.Block(H * hd, H, KV, hd, rope_theta=5e5)
+    b.fill_cache(r.standard_normal((KV, T - n_rows, hd)).astype(np.float32),
+                 r.standard_normal((KV, T - n_rows, hd)).astype(np.float32))
+    q, k, v = (r.standard_normal((n_rows, n_ * hd)).astype(np.float32) for n_ in (H, KV, KV))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        b.attention_cached_qkv(q, k, v, threads=1)
+        times.append(time.perf_counter() - t0)
+        b.clear_cache()
+        b.fill_cache(r.standard_normal((KV, T - n_rows, hd)).astype(np.float32),
+                     r.standard_normal((KV, T - n_rows, hd)).astype(np.float32))
+    times.sort()
+    whole = T * (T + 1) // 2
+    part = whole - (T - n_rows) * (T - n_rows + 1) // 2
+    return {"value": round(times[len(times) // 2] * 1e6 * whole / part, 1), "unit": "us/prefill", "cores": 1,
+            "kind": "port", "workload": "llama1b_prefill_t2048",
+            "sample": "the last 64 of the 2048 rows (%.1f %% of the head loop's multiply-adds), median of %d, "
+                      "scaled to the whole prefill; C restatement of the reference's single-threaded Crystal "
+                      "path" % (100.0 * part / whole, reps)}
+
+
 def layer_decode(sa, np, steps):
     """BASELINE configs[0] on the device: one Llama-3.2-1B-shaped attention layer (hidden 2048, 32 Q /
     8 KV heads, head_dim 64), projections included, 512 cached positions, one new row per call, host
@@ -462,6 +494,8 @@ def main():
                                     "unit": "TFLOP/s", "frac": round(p["kernel_tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
                                     "kernel_us": round(p["kernel_us"], 2), "flops_per_launch": p["flops"],
                                     "traffic": load_traffic("prefill_turns_kernel<64, 2>", p["workload"])}
+    if p and not args.no_cpu:
+        line["cpu_baseline_prefill"] = cpu_baseline_prefill()
     if not args.only:
         line["yardsticks"] = yardsticks(torch)
     print(json.dumps(line))
