@@ -652,6 +652,13 @@ int prefill_key_splits(const SeqTable &st, const Shape &sh, int items) {
     longest = t > longest ? t : longest;
   }
   int ns = (int)((512 + wgs - 1) / wgs);
+  // With long key ranges, about 1024 workgroups: four-wavefront workgroups that share the
+  // compute units two or more at a time and drift apart then do better than 512 of eight
+  // wavefronts, one per unit, whose two wavefronts per SIMD move in step (512 rows on 16384
+  // cached, 128 row blocks: 1078 -> 1053 us); chunks under 32 tiles lose more to their set-up
+  // (1024 rows into an empty cache: 109 -> 115 us).
+  const int ns_1024 = (int)((1024 + wgs - 1) / wgs);
+  if (longest / ns_1024 >= 32) ns = ns_1024;
   const int cap = longest / 8;  // at least eight key tiles per chunk
   if (ns > cap) ns = cap;
   if (ns > 16) ns = 16;
