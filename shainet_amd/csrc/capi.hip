@@ -211,6 +211,12 @@ int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
 int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc, float *out, SeqTable &st,
                   const Shape &sh, int total_tokens, float scale, hipStream_t stream, const PrepArgs *prep) {
   const Path path = choose_path(st, sh);
+  // the MFMA prefill kernels address the rows of a (sequence, kv head) by a 32-bit byte offset;
+  // said before anything is written to the cache
+  if (path == Path::kPrefillMfma && (long long)sh.cap * sh.hd * 4 > 0xffffffffLL)
+    return fail(SHAINET_HIP_ERR_ARGUMENT,
+                "capacity %d x head_dim %d x 4 bytes is 4 GiB or more: not supported for more than 16/g new rows",
+                sh.cap, sh.hd);
   hipError_t e;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   if (c->profiling) {
