@@ -753,3 +753,33 @@ def test_prefill_scores_far_from_unit_scale(hip, H, KV, hd, splits, monkeypatch)
             want = blocks[0].attention_cached_qkv(q[lo:hi], k[lo:hi], v[lo:hi], threads=8)
             assert np.isfinite(got).all(), name
             rm.assert_close(got, want, ATOL, RTOL, f"{name} hd={hd} rows {lo}..{hi}")
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_prefill_random_shapes(hip, seed, monkeypatch):
+    """The MFMA prefill kernels over unrelated shapes: both head dims, every group size, one to four
+    sequences with different cached and new lengths in one call (row blocks of one wavefront next to
+    full ones, diagonals at every offset inside a tile), QK-norm and bias on odd seeds, the key range
+    cut into 1 to 4 chunks; two calls, the second on the grown caches."""
+    r0 = np.random.default_rng(2000 + seed)
+    hd = int(r0.choice([64, 128]))
+    KV = int(r0.choice([1, 2, 4]))
+    g = int(r0.choice([1, 2, 3, 4, 8]))
+    B = int(r0.choice([1, 2, 4]))
+    splits = int(r0.choice([0, 0, 2, 3, 4]))
+    if splits:
+        monkeypatch.setenv("SHAINET_HIP_PREFILL_SPLITS", str(splits))
+    cached = [int(x) for x in r0.integers(0, 400, B)]
+    first = [int(x) for x in r0.integers(17, 260, B)]
+    second = [int(x) for x in r0.integers(17, 120, B)]
+    ctx, cache, blocks, r = make_pair(hip, KV * g, KV, hd, 1e6, norm=bool(seed & 1), bias=bool(seed & 1), batch=B,
+                                      capacity=800, seed=seed)
+    for s_, L in enumerate(cached):
+        if L:
+            kf, vf = (r.standard_normal((KV, L, hd)).astype(np.float32) for _ in range(2))
+            cache.fill(s_, kf, vf)
+            blocks[s_].fill_cache(kf, vf)
+    what = f"hd {hd} KV {KV} g {g} B {B} splits {splits} cached {cached}"
+    assert check_step(ctx, cache, blocks, r, first, what=f"{what} new {first}") < 1e-4
+    assert check_step(ctx, cache, blocks, r, second, what=f"{what} then {second}") < 1e-4
+    check_cache_bits(cache, blocks)
