@@ -75,8 +75,10 @@ __device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &
 // G = 1: four wavefronts, each with 32 virtual rows, walk the key tiles together.
 // G = 2: eight wavefronts; wavefronts 4..7 own the same rows as 0..3 and take every
 // second key tile, so that each SIMD holds two wavefronts of one workgroup and the
-// vector-ALU work of one hides behind the MFMAs of the other even when a launch
-// puts a single workgroup on a compute unit.  The two halves merge through LDS.
+// waits of one (barrier, LDS and memory latencies) hide behind the work of the other
+// even when a launch puts a single workgroup on a compute unit (vector instructions
+// do not hide: fp32 MFMAs and vector instructions share the SIMD's lanes).  The two
+// halves merge through LDS.
 // One workgroup's work: the row block (and key chunk) number `bid` of the launch.
 template <int HD, bool SPLIT, int G>
 __device__ __forceinline__ void prefill_block(const int bid, const float *__restrict__ q_rot,
@@ -257,8 +259,8 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
 
   // Software pipeline over the key tiles, in steps of G tiles (one per group of
   // wavefronts; below "tile sp" is this group's tile of step sp).  Step sp issues the
-  // MFMAs of S^T(sp+1) before the softmax arithmetic of tile sp, so the vector ALU
-  // works in their shadow, then O^T += V^T(sp) P^T(sp).  K runs two steps ahead of V:
+  // MFMAs of S^T(sp+1) before the softmax arithmetic of tile sp (its scores are then a
+  // step old and certainly there), then O^T += V^T(sp) P^T(sp).  K runs two steps ahead of V:
   //   LDS at the start of step sp:  K(sp+1) in Ks[(sp+1)&1], V(sp) in Vs[sp&1];
   //   registers:                     K(sp+2), V(sp+1), fetched during step sp-1.
   // The step first parks those registers in the two LDS stages nobody reads any
