@@ -195,13 +195,13 @@ def cpu_baseline(w, reps):
 
 def cpu_baseline_prefill(reps=3):
     """The oracle, one thread, on a bounded part of the 2048-row causal prefill of the Llama-3.2-1B
-    shape: its last 64 rows on top of the 1984 rows before them, extrapolated to the whole prefill
+    shape: its last 256 rows on top of the 1792 rows before them, extrapolated to the whole prefill
     by the multiply-adds of the head loop (the scalar path's time is proportional to them)."""
     import numpy as np
 
     from oracle import oracle as orc
 
-    H, KV, hd, T, n_rows = 32, 8, 64, 2048, 64
+    H, KV, hd, T, n_rows = 32, 8, 64, 2048, 256
     r = np.random.default_rng(4)
     b = orc.Block(H * hd, H, KV, hd, rope_theta=5e5)
     b.fill_cache(r.standard_normal((KV, T - n_rows, hd)).astype(np.float32),
@@ -220,9 +220,9 @@ def cpu_baseline_prefill(reps=3):
     part = whole - (T - n_rows) * (T - n_rows + 1) // 2
     return {"value": round(times[len(times) // 2] * 1e6 * whole / part, 1), "unit": "us/prefill", "cores": 1,
             "kind": "port", "workload": "llama1b_prefill_t2048",
-            "sample": "the last 64 of the 2048 rows (%.1f %% of the head loop's multiply-adds), median of %d, "
+            "sample": "the last %d of the 2048 rows (%.1f %% of the head loop's multiply-adds), median of %d, "
                       "scaled to the whole prefill; C restatement of the reference's single-threaded Crystal "
-                      "path" % (100.0 * part / whole, reps)}
+                      "path" % (n_rows, 100.0 * part / whole, reps)}
 
 
 def layer_decode(sa, np, steps):
@@ -415,10 +415,10 @@ def main():
     results[head.name] = head.run_decode(K, W)
     cpu = None
     if not args.no_cpu:
-        cpu_us = cpu_baseline(head, 5)
+        cpu_us = cpu_baseline(head, 21)
         cpu = {"value": cpu_us, "unit": "us/layer-step", "cores": 1, "kind": "port",
                "sample": "one decode layer-step of the headline workload (16 sequences, same cache), "
-                         "median of 5, C restatement of the reference's single-threaded Crystal path",
+                         "median of 21, C restatement of the reference's single-threaded Crystal path",
                "host_cores_visible": os.cpu_count()}
     head.close()
 
