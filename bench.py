@@ -27,6 +27,36 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3
+MIN_WARMUP_S = 0.06         # every workload is warmed up for at least this long (and --warmup steps)
+
+# The seeded cached lengths of the headline workload: 16 draws from U[2048, 8192]
+def headline_lengths():
+    import numpy as np
+
+    return [int(x) for x in np.random.default_rng(2024).integers(2048, 8193, 16)]
+
+
+# name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence (None = the headline's)
+HEADLINE = ("qwen3_8b_decode_b16_ctx2048-8192", 32, 8, 128, 1e6, True, None)
+DECODE_WORKLOADS = [
+    ("llama1b_decode_b1_ctx1024", 32, 8, 64, 5e5, False, [1024]),
+    ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096]),
+    ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384]),
+    ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4),
+    # the headline shape with every sequence near the top of its length range (1.07 GB per step)
+    ("qwen3_8b_decode_b16_ctx8192", 32, 8, 128, 1e6, True, [7936] * 16),
+]
+# name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence, new rows per sequence
+PREFILL_WORKLOADS = [
+    ("llama1b_prefill_t2048", 32, 8, 64, 5e5, False, [0], 2048),
+    ("llama1b_prefill_t8192", 32, 8, 64, 5e5, False, [0], 8192),
+    ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512),
+    # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
+    ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048),
+    # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
+    # through the split-K decode kernel as further columns of its tiles)
+    ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, None, 4),
+]
 
 
 def decode_bytes(KV, hd, visible):
@@ -78,9 +108,8 @@ class Workload:
     def run_decode(self, steps, warmup):
         """Consecutive decode steps appending to the cache."""
         torch, ctx = self.torch, self.ctx
-        total = warmup + 2 * steps
-        self.alloc(total + 1)
-        q, k, v, out = self.rows(min(total, 64))
+        self.alloc(2 * steps + 1)
+        q, k, v, out = self.rows(min(2 * steps, 64))
         nt = [1] * self.B
         n = q.shape[0]
         # the timed loop holds nothing but the C call: the row sets are bound beforehand
@@ -89,23 +118,34 @@ class Workload:
         def step(i):
             calls[i % n]()
 
-        for i in range(warmup):
-            step(i)
-        ctx.sync()
+        # Warm-up: at least `warmup` steps and at least MIN_WARMUP_S of them, in runs of `steps`
+        # steps after each of which the caches are cut back to their starting lengths (the timed
+        # steps then see exactly the lengths of the workload's name).  A handful of 0.1 ms
+        # launches after an idle stretch run on a device that has not reached the clocks and power
+        # state it then holds: measured that way, the same kernel is 3 to 15 % slower.
+        t_w, n_w = time.perf_counter(), 0
+        while n_w < warmup or time.perf_counter() - t_w < MIN_WARMUP_S:
+            for i in range(steps):
+                step(i)
+            n_w += steps
+            ctx.sync()
+            for s, L in enumerate(self.lens):
+                self.cache.truncate(s, L)
+        warm_ms = (time.perf_counter() - t_w) * 1e3
         t0 = time.perf_counter()
         for i in range(steps):
-            step(warmup + i)
+            step(i)
         ctx.sync()
         wall = time.perf_counter() - t0
         # second pass with HIP events around the split-K kernel only
         ctx.profile(True)
         for i in range(steps):
-            step(warmup + steps + i)
+            step(steps + i)
         samples = ctx.profile_samples(steps + 8)
         k_ms, launches = float(samples.sum()), len(samples)
         ctx.profile(False)
-        vis_wall = [[L + warmup + i + 1 for L in self.lens] for i in range(steps)]
-        vis_prof = [[L + warmup + steps + i + 1 for L in self.lens] for i in range(steps)]
+        vis_wall = [[L + i + 1 for L in self.lens] for i in range(steps)]
+        vis_prof = [[L + steps + i + 1 for L in self.lens] for i in range(steps)]
         b_wall = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_wall) / steps
         b_prof = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_prof) / steps
         us = wall / steps * 1e6
@@ -115,8 +155,9 @@ class Workload:
         pct = [float(x) * 1e3 for x in np.percentile(samples, (10, 50, 90))] if launches else [0.0] * 3
         return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "kernel_us_p10": pct[0],
                 "kernel_us_p50": pct[1], "kernel_us_p90": pct[2], "launches": launches,
+                "warmup_launches": n_w, "warmup_ms": warm_ms,
                 "bytes_per_step": b_wall, "step_gbps": b_wall / us / 1e3, "kernel_gbps": b_prof / kus / 1e3,
-                "kernel_bytes": b_prof}
+                "kernel_bytes": b_prof, "frac_of_hbm_peak": b_prof / kus / 1e3 / HBM_PEAK_GBPS}
 
     def run_prefill(self, steps, warmup):
         """T new rows on top of S cached ones; the cache is truncated back between steps."""
@@ -134,12 +175,13 @@ class Workload:
         # then holds only after some tens of milliseconds of matrix work (the first launches of
         # T = 2048 take 183 us, later ones 165 us)
         t_w, n_w = time.perf_counter(), 0
-        while n_w < warmup or time.perf_counter() - t_w < 0.06:
+        while n_w < warmup or time.perf_counter() - t_w < MIN_WARMUP_S:
             step()
             n_w += 1
             if n_w % 4 == 0:
                 ctx.sync()
         ctx.sync()
+        warm_ms = (time.perf_counter() - t_w) * 1e3
         t0 = time.perf_counter()
         for _ in range(steps):
             step()
@@ -154,8 +196,9 @@ class Workload:
         us = wall / steps * 1e6
         kus = k_ms / max(launches, 1) * 1e3
         return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "launches": launches,
-                "warmup_launches": n_w, "flops": fl,
-                "step_tflops": fl / us / 1e6, "kernel_tflops": fl / kus / 1e6}
+                "warmup_launches": n_w, "warmup_ms": warm_ms, "flops": fl,
+                "step_tflops": fl / us / 1e6, "kernel_tflops": fl / kus / 1e6,
+                "frac_of_mfma_peak": fl / kus / 1e6 / FP32_MFMA_PEAK_TFLOPS}
 
     def close(self):
         if self.cache is not None:
@@ -297,6 +340,20 @@ def model_decode(sa, np, steps, ctx_len=512):
             "prefill_tflops": 2.0 * (weight_bytes / 4 - d * V) * ctx_len / prefill_s / 1e12}
 
 
+# The kernels the two roofline objects of the bench line price, and the workloads they are priced on.
+ROOFLINE_KERNELS = {
+    "roofline": ("decode_splitk_kernel<128, 4>", "qwen3_8b_decode_b16_ctx2048-8192"),
+    "roofline_prefill": ("prefill_turns_kernel<64, 2>", "llama1b_prefill_t2048"),
+}
+
+
+def profile_file(kernel, workload):
+    """Name of the rocprofv3 summary under profiles/ that covers a kernel on a workload."""
+    import re
+
+    return re.sub(r"[^A-Za-z0-9]+", "_", kernel).strip("_") + "_" + workload + ".md"
+
+
 def load_traffic(kernel, workload, bytes_per_launch=None):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), kept as a
     committed summary; None until measured.  The decode launches of the counter runs are the first
@@ -404,14 +461,15 @@ def main():
 
     K, W = args.steps, args.warmup
     only = set(filter(None, args.only.split(",")))
-    lens3 = [int(x) for x in np.random.default_rng(2024).integers(2048, 8193, 16)]
+    lens3 = headline_lengths()
     results = {}
 
     def want(name):
         return not only or name in only
 
     # headline: configs[2]
-    head = Workload(sa, torch, "qwen3_8b_decode_b16_ctx2048-8192", 32, 8, 128, 1e6, True, lens3, 1, 3)
+    name, H, KV, hd, th, norm, _ = HEADLINE
+    head = Workload(sa, torch, name, H, KV, hd, th, norm, lens3, 1, 3)
     results[head.name] = head.run_decode(K, W)
     cpu = None
     if not args.no_cpu:
@@ -422,34 +480,18 @@ def main():
                "host_cores_visible": os.cpu_count()}
     head.close()
 
-    small = max(10, K // 4)
-    decode_cfgs = [
-        ("llama1b_decode_b1_ctx1024", 32, 8, 64, 5e5, False, [1024], K),
-        ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096], K),
-        ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384], K),
-        ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4, K),
-        # the headline shape with every sequence at the top of its length range (1.07 GB per step)
-        ("qwen3_8b_decode_b16_ctx8192", 32, 8, 128, 1e6, True, [8192 - K - W - 8] * 16, max(20, K // 2)),
-    ]
-    for name, H, KV, hd, th, norm, lens, k_ in decode_cfgs:
+    for name, H, KV, hd, th, norm, lens in DECODE_WORKLOADS:
         if want(name):
             w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, 1, 5)
-            results[name] = w.run_decode(k_, W)
+            results[name] = w.run_decode(K if len(lens) < 16 else max(20, K // 2), W)
             w.close()
-    prefill_cfgs = [
-        ("llama1b_prefill_t2048", 32, 8, 64, 5e5, False, [0], 2048, K),
-        ("llama1b_prefill_t8192", 32, 8, 64, 5e5, False, [0], 8192, max(5, K // 20)),
-        ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512, max(5, K // 10)),
-        # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
-        ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048, max(5, K // 2)),
-        # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
-        # through the split-K decode kernel as further columns of its tiles)
-        ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, lens3, 4, small),
-    ]
-    for name, H, KV, hd, th, norm, lens, T, k_ in prefill_cfgs:
+    fewer = {"llama1b_prefill_t2048": K, "llama1b_prefill_t8192": max(5, K // 20),
+             "qwen3_30b_chunked_prefill_t512_on_16384": max(5, K // 10), "qwen3_8b_prefill_t2048": max(5, K // 2),
+             "qwen3_8b_decode_b16_4rows_ctx2048-8192": max(10, K // 4)}
+    for name, H, KV, hd, th, norm, lens, T in PREFILL_WORKLOADS:
         if want(name):
-            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, T, 7)
-            results[name] = w.run_prefill(k_, max(2, W // 4))
+            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens3 if lens is None else lens, T, 7)
+            results[name] = w.run_prefill(fewer[name], max(2, W // 4))
             w.close()
 
     if want("llama1b_layer_decode_ctx512"):
@@ -475,13 +517,15 @@ def main():
         "config": {"workload": head.name, "num_heads": 32, "num_kv_heads": 8, "head_dim": 128, "qk_norm": True,
                    "rope_theta": 1e6, "batch": 16, "cached_lengths": lens3, "new_rows_per_sequence": 1},
         "hbm_gbps": round(h["step_gbps"], 1),
-        "roofline": {"bound": "hbm", "kernel": "decode_splitk_kernel<128, 4>", "achieved": round(h["kernel_gbps"], 1),
+        "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNELS["roofline"][0], "achieved": round(h["kernel_gbps"], 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(h["kernel_gbps"] / HBM_PEAK_GBPS, 4),
                      "kernel_us": round(h["kernel_us"], 2), "kernel_us_p10_p50_p90": [round(h["kernel_us_p10"], 2),
                                                                                       round(h["kernel_us_p50"], 2),
                                                                                       round(h["kernel_us_p90"], 2)],
                      "bytes_per_launch": int(h["kernel_bytes"]),
-                     "traffic": load_traffic("decode_splitk_kernel<128, 4>", head.name, h["kernel_bytes"])},
+                     "warmup_ms": round(h["warmup_ms"], 1), "warmup_launches": h["warmup_launches"],
+                     "profile": "profiles/" + profile_file(*ROOFLINE_KERNELS["roofline"]),
+                     "traffic": load_traffic(ROOFLINE_KERNELS["roofline"][0], head.name, h["kernel_bytes"])},
         "cpu_baseline": cpu,
         "workloads": {k_: {kk: (round(vv, 3) if isinstance(vv, float) else vv) for kk, vv in r.items()
                            if kk != "workload"} for k_, r in results.items()},
@@ -489,11 +533,14 @@ def main():
     p = results.get("llama1b_prefill_t2048")
     if p:
         line["prefill_tflops"] = round(p["step_tflops"], 2)
-        line["roofline_prefill"] = {"bound": "mfma", "kernel": "prefill_turns_kernel<64, 2>", "workload": p["workload"],
+        line["roofline_prefill"] = {"bound": "mfma", "kernel": ROOFLINE_KERNELS["roofline_prefill"][0],
+                                    "workload": p["workload"],
                                     "achieved": round(p["kernel_tflops"], 2), "peak": FP32_MFMA_PEAK_TFLOPS,
                                     "unit": "TFLOP/s", "frac": round(p["kernel_tflops"] / FP32_MFMA_PEAK_TFLOPS, 4),
                                     "kernel_us": round(p["kernel_us"], 2), "flops_per_launch": p["flops"],
-                                    "traffic": load_traffic("prefill_turns_kernel<64, 2>", p["workload"])}
+                                    "warmup_ms": round(p["warmup_ms"], 1), "warmup_launches": p["warmup_launches"],
+                                    "profile": "profiles/" + profile_file(*ROOFLINE_KERNELS["roofline_prefill"]),
+                                    "traffic": load_traffic(ROOFLINE_KERNELS["roofline_prefill"][0], p["workload"])}
     if p and not args.no_cpu:
         line["cpu_baseline_prefill"] = cpu_baseline_prefill()
     if not args.only:

@@ -156,6 +156,26 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
  * and QK-norm of Q exactly (llama_block.cr:332-344). */
 int shainet_attn_last_q_rot(shainet_attn_ctx *ctx, float *out, int rows);
 
+/* What a shainet_attn_forward call with these sequences (cached positions start_pos[s], new rows
+ * new_tokens[s]) launches for its attention step, without launching anything; needs no device.
+ * plan[0] path: 0 = split-K decode kernel, 1 = MFMA prefill kernel, 2 = generic kernel;
+ * plan[1] head_dim; plan[2] key chunks per row block (1 = none, > 1 adds the combine kernel);
+ * plan[3] wavefront groups per workgroup (1 = four wavefronts, 2 = eight); plan[4] row blocks a
+ * workgroup takes in turn (0 = one workgroup per block and chunk); plan[5] workgroups;
+ * plan[6] decode: 16-key tiles per workgroup, prefill: row blocks; plan[7] workgroups per
+ * compute unit the launch is held to (0 = no limit).  Lets a test name the kernel instantiation
+ * it covers.  No counterpart in the reference, whose kernel has one shape (cuda_kernels.cu:808-825). */
+int shainet_attn_describe_plan(int num_heads, int num_kv_heads, int head_dim, int n_seqs, const int *start_pos,
+                               const int *new_tokens, int plan[8]);
+
+/* RoPE.apply (src/shainet/transformer/rope.cr:7-33): x and out are [seq_len, head_dim] rows;
+ * row r is rotated by (r + start_pos) * theta^(-2i/head_dim), half-split pairs (i, i + head_dim/2),
+ * everything in fp64 on the device and rounded to fp32 once, an odd trailing column copied
+ * through.  LlamaBlock does not call it (its own RoPE keeps the angle in fp32,
+ * llama_block.cr:274-277); it is the stand-alone module function that spec/rope_kv_cache_spec.cr:4-27
+ * pins.  mem = HOST: synchronous; DEVICE: asynchronous on the default stream. */
+int shainet_rope_apply(const float *x, float *out, int seq_len, int head_dim, int start_pos, double theta, int mem);
+
 /* ---- the attention half of a LlamaBlock, weights included ------------------
  *
  * State and behaviour of src/shainet/transformer/llama_block.cr for

@@ -671,12 +671,44 @@ size_t prefill_partial_floats(const Shape &sh, int items, int ns) {
   return ns > 1 ? (size_t)items * sh.KV * ns * 128 * (sh.hd + 2) : 0;
 }
 
+PrefillLaunch plan_prefill_launch(const Shape &sh, int items, int ns, int wgs_per_cu, int groups) {
+  PrefillLaunch p;
+  p.n_wgs = (long long)items * sh.KV * ns;
+  // With fewer workgroups than three per compute unit everything is resident at
+  // once: run one workgroup per compute unit (below) and give it eight wavefronts,
+  // two per SIMD (G = 2).  Larger launches already have several workgroups per unit.
+  p.groups = groups == 1 || groups == 2 ? groups : (p.n_wgs <= 768 ? 2 : 1);
+  // static LDS of the kernel: two stages of `groups` padded K tiles and V tiles
+  const size_t static_lds = (size_t)2 * p.groups * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
+  p.pad = 0;
+  // With fewer workgroups than three per compute unit everything is resident at
+  // once and the dispatcher cannot balance the triangular work: one workgroup per
+  // compute unit lets it hand the short row blocks to whichever unit finishes first.
+  if (wgs_per_cu == 0 && p.n_wgs <= 768) wgs_per_cu = 1;
+  p.wgs_per_cu = wgs_per_cu >= 1 && wgs_per_cu <= 3 ? wgs_per_cu : 0;
+  if (p.wgs_per_cu) {
+    const size_t want = (size_t)160 * 1024 / wgs_per_cu;  // one more workgroup would not fit
+    const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
+    if (static_lds < floor_ && floor_ <= want) p.pad = floor_ - static_lds;
+  }
+  static const bool turns_off = getenv("SHAINET_HIP_PREFILL_NO_TURNS") != nullptr;
+  // Turns only when the blocks fill them: otherwise compute units would stand idle where the
+  // dispatcher's own hand-out keeps them busy (12 % slower at 640 blocks)
+  const int turns = (int)((p.n_wgs + 255) / 256);
+  p.turns = !turns_off && ns == 1 && p.groups == 2 && p.n_wgs > 256 && p.n_wgs <= 768 &&
+                    p.n_wgs * 100 >= (long long)turns * 256 * 97
+                ? turns
+                : 0;
+  return p;
+}
+
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                           const SeqTable &st, const Shape &sh, int items, int ns, float scale,
-                          hipStream_t stream, int wgs_per_cu, hipEvent_t before, hipEvent_t after) {
+                          hipStream_t stream, int wgs_per_cu, int groups_wanted, hipEvent_t before, hipEvent_t after) {
   if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1 || ns < 1 || (ns > 1 && !partials))
     return hipErrorInvalidValue;
-  const long long n_wgs = (long long)items * sh.KV * ns;
+  const PrefillLaunch plan = plan_prefill_launch(sh, items, ns, wgs_per_cu, groups_wanted);
+  const long long n_wgs = plan.n_wgs;
   if (n_wgs > 0x7fffffffLL) return hipErrorInvalidValue;
   // the kernels address a row of a (sequence, kv head) by a 32-bit byte offset from its first row
   if ((long long)sh.cap * sh.hd * 4 > 0xffffffffLL) return hipErrorInvalidValue;
@@ -684,28 +716,10 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
   dim3 grid((unsigned)n_wgs);
   float *part_o = partials;
   float *part_ml = partials ? partials + (size_t)items * sh.KV * ns * 128 * sh.hd : nullptr;
-  // With fewer workgroups than three per compute unit everything is resident at
-  // once: run one workgroup per compute unit (below) and give it eight wavefronts,
-  // two per SIMD (G = 2).  Larger launches already have several workgroups per unit.
-  static const int groups_env = getenv("SHAINET_HIP_PREFILL_GROUPS") ? atoi(getenv("SHAINET_HIP_PREFILL_GROUPS")) : 0;
-  const int groups = groups_env == 1 || groups_env == 2 ? groups_env : (n_wgs <= 768 ? 2 : 1);
-  // static LDS of the kernel: two stages of `groups` padded K tiles and V tiles
-  const size_t static_lds = (size_t)2 * groups * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
-  size_t pad = 0;
-  // With fewer workgroups than three per compute unit everything is resident at
-  // once and the dispatcher cannot balance the triangular work: one workgroup per
-  // compute unit lets it hand the short row blocks to whichever unit finishes first.
-  if (wgs_per_cu == 0 && n_wgs <= 768) wgs_per_cu = 1;
-  if (wgs_per_cu >= 1 && wgs_per_cu <= 3) {
-    const size_t want = (size_t)160 * 1024 / wgs_per_cu;  // one more workgroup would not fit
-    const size_t floor_ = (size_t)160 * 1024 / (wgs_per_cu + 1) + 256;
-    if (static_lds < floor_ && floor_ <= want) pad = floor_ - static_lds;
-  }
-  static const bool turns_off = getenv("SHAINET_HIP_PREFILL_NO_TURNS") != nullptr;
-  // (only when the blocks fill those turns: otherwise compute units would stand idle where the
-  // dispatcher's own hand-out keeps them busy, 12 % slower at 640 blocks)
-  const int turns = (int)((n_wgs + 255) / 256);
-  if (!turns_off && ns == 1 && groups == 2 && n_wgs > 256 && n_wgs <= 768 && n_wgs * 100 >= (long long)turns * 256 * 97) {
+  const int groups = plan.groups;
+  const size_t pad = plan.pad;
+  if (plan.turns) {
+    const int turns = plan.turns;
     dim3 fewer((unsigned)((n_wgs + turns - 1) / turns));
     if (sh.hd == 64)
       SHAINET_LAUNCH_TIMED((prefill_turns_kernel<64, 2>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, vc, out,

@@ -111,10 +111,20 @@ int prefill_key_splits(const SeqTable &st, const Shape &sh, int items);
 size_t prefill_partial_floats(const Shape &sh, int items, int ns);
 // wgs_per_cu: 0 = default; 1..3 pads the kernel's LDS so that at most that many
 // workgroups share a compute unit (a tuning knob).
+// groups: 0 = default; 1 or 2 forces the number of wavefront groups per workgroup (a tuning knob).
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                           const SeqTable &st, const Shape &sh, int items, int ns, float scale,
-                          hipStream_t stream, int wgs_per_cu = 0, hipEvent_t before = nullptr,
+                          hipStream_t stream, int wgs_per_cu = 0, int groups = 0, hipEvent_t before = nullptr,
                           hipEvent_t after = nullptr);
+// Which instantiation a prefill launch uses and how it is laid out; launch_prefill follows it.
+struct PrefillLaunch {
+  long long n_wgs;   // row blocks x kv heads x key chunks
+  int groups;        // 1: four wavefronts per workgroup; 2: eight
+  int turns;         // 0: one workgroup per row block and chunk; 2 or 3: prefill_turns_kernel with that many blocks per workgroup
+  int wgs_per_cu;    // 0: as the kernel's registers and LDS allow; 1..3: LDS padded to that occupancy
+  size_t pad;        // bytes of dynamic LDS that enforce wgs_per_cu
+};
+PrefillLaunch plan_prefill_launch(const Shape &sh, int items, int ns, int wgs_per_cu, int groups);
 hipError_t launch_generic(const float *q_rot, const float *kc, const float *vc, float *out,
                           const SeqTable &st, const Shape &sh, int total_tokens, float scale,
                           hipStream_t stream);
@@ -164,11 +174,13 @@ struct GemvPlan {
 GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim = 0);
 hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
 
-// One pinned host int for the whole library that kernels set when they give up a bounded
-// wait for other workgroups (null when it cannot be allocated); check_error_word, called
-// after a wait for a stream, turns a set word into SHAINET_HIP_ERR_RUNTIME and clears it.
-int *error_word();
-int check_error_word();
+// A pinned host int per context (block, model) that its kernels set when they give up a
+// bounded wait for other workgroups (null when it cannot be allocated); check_error_word,
+// called after a wait for the handle's stream, turns a set word into SHAINET_HIP_ERR_RUNTIME
+// and clears it: the give-up is reported by the handle whose kernel gave up.
+int *alloc_error_word();
+void free_error_word(int *w);
+int check_error_word(int *w);
 
 hipError_t launch_legacy_append(const float *staging, float *kc, float *vc, int new_tokens, int start_pos,
                                 int num_kv_heads, int head_dim, int capacity, hipStream_t stream);

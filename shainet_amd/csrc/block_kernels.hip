@@ -237,6 +237,30 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const float *__restrict
   }
 }
 
+// RoPE.apply (rope.cr:7-33): one lane per (row, pair).  Everything in fp64 as the reference has
+// it (Float32 operands widened, `theta ** (2.0 * i / head_dim)`, the angle, Math.cos / Math.sin,
+// both products and their difference or sum), rounded once when the result is stored.
+__global__ __launch_bounds__(256) void rope_apply_kernel(const float *__restrict__ x, float *__restrict__ out,
+                                                         int seq_len, int head_dim, int start_pos, double theta) {
+  const int half = head_dim / 2;
+  const long long per_row = half + (head_dim & 1);  // the odd trailing column rides along as one more item
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)seq_len * per_row) return;
+  const int pos = (int)(idx / per_row), i = (int)(idx - (long long)pos * per_row);
+  const float *xr = x + (long long)pos * head_dim;
+  float *orow = out + (long long)pos * head_dim;
+  if (i == half) {
+    orow[head_dim - 1] = xr[head_dim - 1];
+    return;
+  }
+  const double freq = 1.0 / pow(theta, 2.0 * (double)i / (double)head_dim);
+  const double angle = (double)(pos + start_pos) * freq;
+  const double c = cos(angle), s = sin(angle);
+  const double x0 = (double)xr[i], x1 = (double)xr[i + half];
+  orow[i] = (float)(x0 * c - x1 * s);
+  orow[i + half] = (float)(x1 * c + x0 * s);
+}
+
 }  // namespace
 
 hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
@@ -278,6 +302,17 @@ hipError_t launch_repetition_penalty(float *logits, int vocab, const int *ids, i
                                      hipStream_t stream) {
   if (n < 1) return hipSuccess;
   hipLaunchKernelGGL(repetition_penalty_kernel, dim3(1), dim3(64), 0, stream, logits, vocab, ids, n, penalty);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_apply(const float *x, float *out, int seq_len, int head_dim, int start_pos, double theta,
+                             hipStream_t stream) {
+  if (!x || !out || seq_len < 0 || head_dim < 1) return hipErrorInvalidValue;
+  const long long items = (long long)seq_len * (head_dim / 2 + (head_dim & 1));
+  if (items == 0) return hipSuccess;
+  if ((items + 255) / 256 > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, x, out, seq_len,
+                     head_dim, start_pos, theta);
   return hipGetLastError();
 }
 

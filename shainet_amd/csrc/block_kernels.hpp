@@ -23,6 +23,12 @@ hipError_t launch_add_bias_row(float *logits, const float *bias, int n, hipStrea
 hipError_t launch_repetition_penalty(float *logits, int vocab, const int *ids, int n, double penalty,
                                      hipStream_t stream);
 
+// RoPE.apply (rope.cr:7-33) on [seq_len, head_dim] rows: half-split rotation by
+// (row + start_pos) * theta^(-2i/head_dim), frequency, angle, cosine, sine and the products in
+// fp64, one rounding to fp32; an odd trailing column is copied through.
+hipError_t launch_rope_apply(const float *x, float *out, int seq_len, int head_dim, int start_pos, double theta,
+                             hipStream_t stream);
+
 // Top-k of a logits row, descending by value, ties by ascending index, NaN never
 // selected (Sampler#sample's selection); with finite_only also +-inf are skipped
 // (Sampler.greedy).  scratch: topk_scratch_bytes(vocab, k) bytes.  out_ids /

@@ -11,6 +11,7 @@
 
 #include "../../include/shainet_hip_attn.h"
 #include "attn_kernels.hpp"
+#include "block_kernels.hpp"
 
 using namespace shainet;
 
@@ -33,24 +34,24 @@ void shainet_hip_set_error(int code, const char *msg) { fail(code, "%s", msg); }
 
 namespace shainet {
 
-int *error_word() {
-  static int *word = [] {
-    int *p = nullptr;
-    if (hipHostMalloc((void **)&p, sizeof(int), hipHostMallocPortable) != hipSuccess) {
-      (void)hipGetLastError();
-      return (int *)nullptr;
-    }
-    *p = 0;
-    return p;
-  }();
-  return word;
+int *alloc_error_word() {
+  int *p = nullptr;
+  if (hipHostMalloc((void **)&p, sizeof(int), hipHostMallocPortable) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  *p = 0;
+  return p;
 }
 
-int check_error_word() {
-  int *w = error_word();
+void free_error_word(int *w) {
+  if (w) (void)hipHostFree(w);
+}
+
+int check_error_word(int *w) {
   if (!w || *(volatile int *)w == 0) return SHAINET_HIP_OK;
   *(volatile int *)w = 0;
-  return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups; the results of the calls since the last wait are invalid and their contexts must be destroyed");
+  return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups; the results of the calls on this handle since its last wait are invalid and it must be destroyed");
 }
 
 }  // namespace shainet
@@ -113,10 +114,14 @@ struct shainet_attn_ctx {
   unsigned *part_flag = nullptr;
   size_t part_flag_cap = 0;
   bool test_lose_marks = false;  // SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS: exercises the give-up path
+  // pinned host word this context's kernels set when they give up a bounded wait; `error` is
+  // the one in use: the context's own, or the one of the block or model that owns the context
+  int *error = nullptr, *own_error = nullptr;
   int last_rows = 0;
   int decode_wgs_override = 0;  // 0 = default workgroup count of the decode split
   int prefill_wgs_per_cu = 0;   // 0 = default occupancy of the prefill kernel
   int prefill_splits_override = 0;  // 0 = default number of key splits of the prefill kernel
+  int prefill_groups_override = 0;  // 0 = default number of wavefront groups of the prefill kernel
   bool profiling = false;
   std::vector<hipEvent_t> prof_events;  // start, stop, start, stop, ...
 };
@@ -186,7 +191,10 @@ Shape shape_of(const shainet_attn_ctx *c, int cap) {
 
 // Zero-initialised flag words of the decode split.
 int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
-  if (!error_word()) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+  if (!c->error) {  // the handle-less context of the reference-named entry points gets its word here
+    c->error = c->own_error = alloc_error_word();
+    if (!c->error) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+  }
   if (n <= c->part_flag_cap) return SHAINET_HIP_OK;
   size_t want = c->part_flag_cap ? c->part_flag_cap : 1024;
   while (want < n) want *= 2;
@@ -239,7 +247,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     d.out = out;
     d.partials = c->partials.p;
     d.part_flag = c->part_flag;
-    d.error = error_word();
+    d.error = c->error;
     d.flag_set = c->test_lose_marks ? c->part_flag + c->part_flag_cap : nullptr;
     d.spin_limit = c->test_lose_marks ? 2000 : 0;
     if (prep) {
@@ -258,7 +266,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
       int rc = c->partials.reserve(prefill_partial_floats(sh, items, ns));
       if (rc) return rc;
       e = launch_prefill(q_rot, kc, vc, out, c->partials.p, st, sh, items, ns, scale, stream,
-                         c->prefill_wgs_per_cu, ev0, ev1);
+                         c->prefill_wgs_per_cu, c->prefill_groups_override, ev0, ev1);
     } else {
       plan_work(st, sh, path);
       if (ev0) (void)hipEventRecord(ev0, stream);
@@ -368,10 +376,13 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
   c->test_lose_marks = getenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS") != nullptr;
   if (const char *env = getenv("SHAINET_HIP_PREFILL_WGS_PER_CU")) c->prefill_wgs_per_cu = atoi(env);
   if (const char *env = getenv("SHAINET_HIP_PREFILL_SPLITS")) c->prefill_splits_override = atoi(env);
+  if (const char *env = getenv("SHAINET_HIP_PREFILL_GROUPS")) c->prefill_groups_override = atoi(env);
   int rc = SHAINET_HIP_OK;
   hipError_t e = hipStreamCreateWithFlags(&c->own_stream, hipStreamNonBlocking);
   if (e != hipSuccess) rc = hip_fail(e, "hipStreamCreate");
   c->stream = c->own_stream;
+  c->error = c->own_error = alloc_error_word();
+  if (!rc && !c->error) rc = fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
   if (!rc) rc = upload(&c->d_q_norm, q_norm, head_dim);
   if (!rc) rc = upload(&c->d_k_norm, k_norm, head_dim);
   if (!rc) rc = ensure_rope_table(c, max_positions > 0 ? max_positions : 1024);
@@ -413,6 +424,7 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
   if (c->part_flag) (void)hipFree(c->part_flag);
   for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
+  free_error_word(c->own_error);
   delete c;
   return SHAINET_HIP_OK;
 }
@@ -420,13 +432,14 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
 int shainet_attn_sync(shainet_attn_ctx *c) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
   HIP_TRY(hipStreamSynchronize(c->stream));
-  return check_error_word();
+  return check_error_word(c->error);
 }
 
 void *shainet_attn_stream(shainet_attn_ctx *c) { return c ? (void *)c->stream : nullptr; }
 
 int shainet_attn_set_stream(shainet_attn_ctx *c, void *stream) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");
+  if ((hipStream_t)stream == c->stream) return SHAINET_HIP_OK;  // nothing changes: no reason to drain the queue
   HIP_TRY(hipStreamSynchronize(c->stream));  // nothing of ours may still run on the old one
   c->stream = (hipStream_t)stream;
   return SHAINET_HIP_OK;
@@ -660,10 +673,17 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   if (mem == SHAINET_HIP_MEM_HOST) {
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
-    return check_error_word();
+    return check_error_word(c->error);
   }
   return SHAINET_HIP_OK;
 }
+
+// The owner of a context (a block, a model) makes the context's kernels report into the owner's
+// word, so that the owner's wait sees what any of its kernels gave up on; null = back to its own.
+void shainet_attn_adopt_error_word(shainet_attn_ctx *c, int *word) {
+  if (c) c->error = word ? word : c->own_error;
+}
+int *shainet_attn_error_word(shainet_attn_ctx *c) { return c ? c->error : nullptr; }
 
 int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, GemvPrep *where) {
   if (!c || !kc || kc->ctx != c || !where)
@@ -714,6 +734,89 @@ int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int 
 }
 
 extern "C" {
+
+int shainet_rope_apply(const float *x, float *out, int seq_len, int head_dim, int start_pos, double theta, int mem) {
+  if (!x || !out || seq_len < 0 || head_dim < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
+  if (mem != SHAINET_HIP_MEM_HOST && mem != SHAINET_HIP_MEM_DEVICE)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "mem must be SHAINET_HIP_MEM_HOST or SHAINET_HIP_MEM_DEVICE");
+  if (seq_len == 0) return SHAINET_HIP_OK;
+  if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  if (mem == SHAINET_HIP_MEM_DEVICE) {
+    const hipError_t e = launch_rope_apply(x, out, seq_len, head_dim, start_pos, theta, nullptr);
+    return e == hipSuccess ? SHAINET_HIP_OK : hip_fail(e, "rope launch");
+  }
+  const size_t bytes = (size_t)seq_len * head_dim * sizeof(float);
+  float *dx = nullptr, *dy = nullptr;
+  hipError_t e = hipMalloc((void **)&dx, bytes);
+  if (e == hipSuccess) e = hipMalloc((void **)&dy, bytes);
+  if (e == hipSuccess) e = hipMemcpy(dx, x, bytes, hipMemcpyHostToDevice);
+  if (e == hipSuccess) e = launch_rope_apply(dx, dy, seq_len, head_dim, start_pos, theta, nullptr);
+  if (e == hipSuccess) e = hipMemcpy(out, dy, bytes, hipMemcpyDeviceToHost);  // waits for the kernel
+  if (dx) (void)hipFree(dx);
+  if (dy) (void)hipFree(dy);
+  return e == hipSuccess ? SHAINET_HIP_OK : hip_fail(e, "shainet_rope_apply");
+}
+
+int shainet_attn_describe_plan(int num_heads, int num_kv_heads, int head_dim, int n_seqs, const int *start_pos,
+                               const int *new_tokens, int plan[8]) {
+  if (!start_pos || !new_tokens || !plan) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!(num_kv_heads > 0 && num_heads > 0 && num_heads % num_kv_heads == 0) || head_dim < 1 || head_dim > 256)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid head geometry");
+  if (n_seqs < 1 || n_seqs > SHAINET_HIP_MAX_BATCH)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", SHAINET_HIP_MAX_BATCH);
+  SeqTable st;
+  memset(&st, 0, sizeof st);
+  st.n_seqs = n_seqs;
+  int total = 0, cap = 1;
+  for (int s = 0; s < n_seqs; ++s) {
+    if (start_pos[s] < 0 || new_tokens[s] < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid sequence");
+    st.slot[s] = s;
+    st.start_pos[s] = start_pos[s];
+    st.n_new[s] = new_tokens[s];
+    st.tok_off[s] = total;
+    total += new_tokens[s];
+    cap = cap > start_pos[s] + new_tokens[s] ? cap : start_pos[s] + new_tokens[s];
+  }
+  st.tok_off[n_seqs] = total;
+  Shape sh;
+  sh.H = num_heads;
+  sh.KV = num_kv_heads;
+  sh.g = num_heads / num_kv_heads;
+  sh.hd = head_dim;
+  sh.cap = cap;
+  sh.seq_stride = (long long)num_kv_heads * cap * head_dim;
+  for (int i = 0; i < 8; ++i) plan[i] = 0;
+  const Path path = choose_path(st, sh);
+  plan[1] = head_dim;
+  if (path == Path::kDecodeSplitK) {
+    SeqTable att;
+    if (!decode_entries(st, sh, att)) return fail(SHAINET_HIP_ERR_RUNTIME, "decode entries do not fit");
+    const DecodePlan p = plan_decode(att, sh, 0);
+    plan[0] = 0;
+    plan[2] = 1;
+    plan[3] = 1;
+    plan[5] = p.n_wgs;
+    plan[6] = p.tiles_per_wg;
+    plan[7] = 1;
+  } else if (path == Path::kPrefillMfma) {
+    const int items = plan_work(st, sh, path);
+    const int ns = prefill_key_splits(st, sh, items);
+    const PrefillLaunch p = plan_prefill_launch(sh, items, ns, 0, 0);
+    plan[0] = 1;
+    plan[2] = ns;
+    plan[3] = p.groups;
+    plan[4] = p.turns;
+    plan[5] = (int)(p.turns ? (p.n_wgs + p.turns - 1) / p.turns : p.n_wgs);
+    plan[6] = items;
+    plan[7] = p.wgs_per_cu;
+  } else {
+    plan[0] = 2;
+    plan[2] = 1;
+    plan[3] = 1;
+    plan[5] = total * num_heads;
+  }
+  return SHAINET_HIP_OK;
+}
 
 int shainet_attn_profile(shainet_attn_ctx *c, int enable) {
   if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "ctx is null");

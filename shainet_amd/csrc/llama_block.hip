@@ -41,6 +41,7 @@ struct shainet_llama_attn {
   shainet_kv_cache *cache = nullptr;
   shainet_kv_cache *scratch_cache = nullptr;  // rows of a no-cache forward call; empty between calls
   int cache_len = 0;  // @cache_len
+  int *shared_error = nullptr;  // the error word of the model that owns this block, if one does
   Projector proj;
   DevF x, qkv, attn, out;
 };
@@ -79,6 +80,8 @@ int ensure_context(shainet_llama_attn *l) {
     return rc;
   }
   l->params_dirty = false;
+  if (l->shared_error) shainet_attn_adopt_error_word(l->ctx, l->shared_error);
+  l->proj.error = shainet_attn_error_word(l->ctx);
   return SHAINET_HIP_OK;
 }
 
@@ -262,7 +265,7 @@ static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_toke
   if (hipMemcpyAsync(out, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
-  return check_error_word();
+  return check_error_word(shainet_attn_error_word(l->ctx));
 }
 
 }  // extern "C"
@@ -346,6 +349,15 @@ int shainet_llama_block_truncate(shainet_llama_block *b, int len) {
   }
   l->cache_len = len;
   return SHAINET_HIP_OK;
+}
+// The model's kernels and its blocks' report a given-up wait into one word, the model's.
+void shainet_llama_block_share_error_word(shainet_llama_block *b, int *word) {
+  shainet_llama_attn *l = b->attn;
+  l->shared_error = word;
+  if (l->ctx) {
+    shainet_attn_adopt_error_word(l->ctx, word);
+    l->proj.error = shainet_attn_error_word(l->ctx);
+  }
 }
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream) {
   int rc = ensure_context(b->attn);
@@ -449,7 +461,7 @@ static int block_forward_any(shainet_llama_block *b, const float *x, int new_tok
   if (hipMemcpyAsync(out, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
-  return check_error_word();
+  return check_error_word(shainet_attn_error_word(b->attn->ctx));
 }
 
 }  // extern "C"

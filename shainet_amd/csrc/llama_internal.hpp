@@ -22,6 +22,10 @@ struct GemvPrep;
 }
 int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, shainet::GemvPrep *where);
 int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out);
+// capi.hip: the pinned host word a context's kernels report a given-up wait into; a block or a
+// model that owns the context makes it the owner's word (null = back to the context's own)
+void shainet_attn_adopt_error_word(shainet_attn_ctx *c, int *word);
+int *shainet_attn_error_word(shainet_attn_ctx *c);
 
 // Device weight buffers of a block / a model, allocated on first request, for a loader
 // that fills them on the device (llama_block.hip, llama_model.hip).
@@ -68,6 +72,8 @@ struct Projector {
   // split products: a word per partial that says when it is complete (zero between launches)
   unsigned *flags = nullptr;
   size_t flags_cap = 0;
+  // where the split products' kernels report a given-up wait: the owner's pinned host word
+  int *error = nullptr;
   // returns a SHAINET_HIP_* status; the message is left for shainet_hip_last_error
   int project(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
               const Fused &f = Fused());

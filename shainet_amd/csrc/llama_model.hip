@@ -22,6 +22,7 @@ using namespace shainet;
 int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out);
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream);
 int shainet_llama_block_truncate(shainet_llama_block *b, int len);
+void shainet_llama_block_share_error_word(shainet_llama_block *b, int *word);
 
 struct shainet_llama_model {
   int vocab = 0, d_model = 0;
@@ -33,6 +34,7 @@ struct shainet_llama_model {
   float *lm_head = nullptr;     // device [d_model, vocab]
   float *lm_bias = nullptr;     // device [vocab] or null
   hipStream_t stream = nullptr;
+  int *error = nullptr;  // pinned host word: set by any kernel of the model that gave up a bounded wait
   Projector proj;
   DevF act[2], logits;
   int *d_tokens = nullptr;
@@ -110,7 +112,7 @@ int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *v
       (vals && hipMemcpyAsync(vals, m->d_vals, k * sizeof(float), hipMemcpyDeviceToHost, m->stream) != hipSuccess) ||
       hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the selection back failed");
-  if (int rc = check_error_word()) return rc;
+  if (int rc = check_error_word(m->error)) return rc;
   *count = host_ids[kMaxTopK];
   for (int i = 0; i < k; ++i) ids[i] = host_ids[i];
   return SHAINET_HIP_OK;
@@ -159,6 +161,8 @@ int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model
   m->vocab = vocab;
   m->d_model = d_model;
   m->eps = eps;
+  m->error = alloc_error_word();  // null without a device: said by the first call that needs one
+  m->proj.error = m->error;
   for (int i = 0; i < n_layers; ++i) {
     shainet_llama_block *b = nullptr;
     int rc = shainet_llama_block_create(&b, d_model, num_heads, ff_hidden, eps, rope_theta, num_kv_heads, head_dim);
@@ -166,6 +170,7 @@ int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model
       shainet_llama_model_destroy(m);
       return rc;
     }
+    shainet_llama_block_share_error_word(b, m->error);
     m->blocks.push_back(b);
   }
   *out = m;
@@ -184,6 +189,7 @@ int shainet_llama_model_destroy(shainet_llama_model *m) {
   m->proj.release();
   for (DevF *f : {&m->act[0], &m->act[1], &m->logits}) f->release();
   if (m->stream) (void)hipStreamDestroy(m->stream);
+  free_error_word(m->error);
   delete m;
   return SHAINET_HIP_OK;
 }
@@ -253,7 +259,7 @@ int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tok
             hipSuccess ||
         hipStreamSynchronize(m->stream) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
-    return check_error_word();
+    return check_error_word(m->error);
   }
   return SHAINET_HIP_OK;
 }
@@ -290,7 +296,7 @@ int shainet_llama_model_generate_greedy(shainet_llama_model *m, int max_tokens, 
     if (hipMemcpyAsync(host_ids, m->d_gen, steps * sizeof(int), hipMemcpyDeviceToHost, m->stream) != hipSuccess ||
         hipStreamSynchronize(m->stream) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "copying the generated ids back failed");
-    if (int rc = check_error_word()) return rc;
+    if (int rc = check_error_word(m->error)) return rc;
     for (int i = 0; i < steps; ++i) {
       bool stop = false;
       for (int j = 0; j < n_stop; ++j) stop = stop || host_ids[i] == stop_ids[j];
@@ -313,7 +319,7 @@ int shainet_llama_model_sync(shainet_llama_model *m) {
   if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
   if (m->stream && hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamSynchronize failed");
-  return check_error_word();
+  return check_error_word(m->error);
 }
 
 int shainet_llama_model_greedy(shainet_llama_model *m, int *token) {
@@ -364,7 +370,7 @@ int shainet_llama_model_read_logits(shainet_llama_model *m, float *logits) {
           hipSuccess ||
       hipStreamSynchronize(m->stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the logits back failed");
-  return check_error_word();
+  return check_error_word(m->error);
 }
 
 }  // extern "C"

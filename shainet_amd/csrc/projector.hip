@@ -297,7 +297,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
       flags = np;
       flags_cap = want;
     }
-    if (p.splits > 1 && !error_word()) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+    if (p.splits > 1 && !error) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "the projector has no error word");
     GemvArgs a = {};
     a.x = xin;
     a.x_stride = xs;
@@ -309,7 +309,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.y = y;
     a.partials = scratch.p;
     a.flags = flags;
-    a.error = error_word();
+    a.error = error;
     a.T = T;
     a.K = K;
     a.N = N;

@@ -73,6 +73,8 @@ _SIGNATURES = {
     "shainet_attn_forward": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_int]),
     "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
+    "shainet_attn_describe_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _i32p, _i32p, _i32p]),
+    "shainet_rope_apply": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_double, C.c_int]),
     "shainet_llama_attn_create": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_int, C.c_int, C.c_int, C.c_double,
                                             C.c_double]),
     "shainet_llama_attn_destroy": (C.c_int, [C.c_void_p]),
@@ -220,6 +222,47 @@ class HIP:
                          scale):
         lib().attention_kv_f32(_ptr(q), _ptr(kc), _ptr(vc), _ptr(out), _ptr(ws), new_tokens, start_pos, num_heads,
                                heads_per_kv, head_dim, capacity, scale)
+
+
+class RoPE:
+    """SHAInet::RoPE (src/shainet/transformer/rope.cr) on the device."""
+
+    @staticmethod
+    def apply(x, start_pos=0, theta=10000.0):
+        """RoPE.apply(x, start_pos, theta): x is [seq_len, head_dim]; numpy in -> numpy out
+        (synchronous), a CUDA torch tensor in -> torch tensor out (default stream)."""
+        import numpy as np
+
+        if hasattr(x, "is_cuda") and x.is_cuda:
+            import torch
+
+            if x.dim() != 2 or x.dtype != torch.float32 or not x.is_contiguous():
+                raise ArgumentError("x must be a contiguous float32 [seq_len, head_dim] tensor")
+            out = torch.empty_like(x)
+            _check(lib().shainet_rope_apply(x.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1], start_pos, theta,
+                                            MEM_DEVICE))
+            return out
+        x = np.ascontiguousarray(x, np.float32)
+        if x.ndim != 2:
+            raise ArgumentError("x must be [seq_len, head_dim]")
+        out = np.empty_like(x)
+        _check(lib().shainet_rope_apply(x.ctypes.data, out.ctypes.data, x.shape[0], x.shape[1], start_pos, theta,
+                                        MEM_HOST))
+        return out
+
+
+PLAN_FIELDS = ("path", "head_dim", "key_chunks", "groups", "turns", "workgroups", "units", "wgs_per_cu")
+PATH_DECODE, PATH_PREFILL, PATH_GENERIC = 0, 1, 2
+
+
+def describe_plan(num_heads, num_kv_heads, head_dim, start_pos, new_tokens):
+    """What the attention step of a forward call with these sequences launches (a dict over
+    PLAN_FIELDS); nothing is launched and no device is needed."""
+    n = len(new_tokens)
+    sp, nt = (C.c_int * n)(*start_pos), (C.c_int * n)(*new_tokens)
+    plan = (C.c_int * 8)()
+    _check(lib().shainet_attn_describe_plan(num_heads, num_kv_heads, head_dim, n, sp, nt, plan))
+    return dict(zip(PLAN_FIELDS, (int(v) for v in plan)))
 
 
 def stream_copy(src, dst, workgroups=4096, stream=None):

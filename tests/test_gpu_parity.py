@@ -8,6 +8,7 @@ import os
 import numpy as np
 import pytest
 
+import prefill_cases as pc
 import refmath as rm
 from oracle import oracle as orc
 
@@ -200,7 +201,7 @@ def test_config2_decode_steps_appending(hip, S):
     kf, vf = (r.standard_normal((KV, S, hd)).astype(np.float32) for _ in range(2))
     cache.fill(0, kf, vf)
     blocks[0].fill_cache(kf, vf)
-    steps = 128 if S == 1024 else 16
+    steps = 128  # BASELINE.json configs[1]: 128 consecutive decode steps at each context length
     worst = max(check_step(ctx, cache, blocks, r, [1], what=f"S={S} step {i}") for i in range(steps))
     assert cache.len(0) == S + steps
     assert worst < 1e-4
@@ -282,7 +283,11 @@ def test_partials_that_never_arrive_are_reported(hip, monkeypatch):
     """Failure handling of the decode split, forced from the host: with the test switch the
     workgroups mark their partials complete in a place nobody looks at and the merging
     workgroups stop polling after 2000 looks, so every kernel still ends by itself; the call
-    that waits for the stream must report it.  A context made without the switch is unaffected."""
+    that waits for the stream must report it.  A context made without the switch is unaffected,
+    and the give-up is reported by the context whose kernel gave up, not by whichever context
+    waits first."""
+    import torch
+
     import shainet_amd as sa
 
     H, KV, hd = 8, 2, 64
@@ -298,6 +303,16 @@ def test_partials_that_never_arrive_are_reported(hip, monkeypatch):
     cache2.fill(0, kf, vf)
     blocks2[0].fill_cache(kf, vf)
     check_step(ctx2, cache2, blocks2, r2, [1])
+    # asynchronous calls on both contexts; the healthy one waits first and must come back clean
+    dev = [torch.from_numpy(a).cuda() for a in rows(r, 1, H, KV, hd)]
+    torch.cuda.synchronize()
+    ctx.forward(cache, *dev, [1])
+    good = ctx2.forward(cache2, *dev, [1])
+    ctx2.sync()
+    assert torch.isfinite(good).all()
+    with pytest.raises(sa.hip.HipError, match="gave up waiting"):
+        ctx.sync()
+    ctx.sync()  # reported once
 
 
 def test_config3_qwen3_8b_batch16_varlen_decode(hip):
@@ -383,21 +398,27 @@ def test_prefill_then_decode_equals_one_prefill(hip):
         assert np.abs(o - outs[0]).max() < 2e-5
 
 
-def test_config4_prefill_2048(hip):
-    H, KV, hd, T = 32, 8, 64, 2048
-    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 500000.0, capacity=T + 64, seed=44)
-    assert check_step(ctx, cache, blocks, r, [T], threads=16) < 1e-4
-    check_step(ctx, cache, blocks, r, [1])
-
-
-def test_config5a_chunked_prefill_on_long_prefix_reduced(hip):
-    # Qwen3-30B-A3B geometry (32 q / 4 kv heads, hd 128, QK-norm); 512 new rows on 4096 cached
-    H, KV, hd, S, T = 32, 4, 128, 4096, 512
-    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=True, capacity=S + T, seed=51)
-    kf, vf = (r.standard_normal((KV, S, hd)).astype(np.float32) for _ in range(2))
-    cache.fill(0, kf, vf)
-    blocks[0].fill_cache(kf, vf)
-    assert check_step(ctx, cache, blocks, r, [T], threads=16) < 1e-4
+@pytest.mark.parametrize("name,H,KV,hd,norm,S,T,inst", pc.CASES, ids=[c[0] for c in pc.CASES])
+def test_prefill_full_size_every_instantiation(hip, name, H, KV, hd, norm, S, T, inst, monkeypatch):
+    """Every instantiation of the MFMA prefill kernels that the planner can pick, each on a shape
+    for which the planner picks it by itself (no tuning variable set), all rows against the
+    oracle.  The table holds BASELINE.json configs[3] (2048 and 8192 rows into an empty cache)
+    and configs[4](a) (512 rows on 16384 cached positions, Qwen3-30B-A3B geometry) at full size."""
+    for var in ("SHAINET_HIP_PREFILL_SPLITS", "SHAINET_HIP_PREFILL_GROUPS", "SHAINET_HIP_PREFILL_WGS_PER_CU",
+                "SHAINET_HIP_PREFILL_NO_TURNS"):
+        monkeypatch.delenv(var, raising=False)
+    plan = hip.describe_plan(H, KV, hd, [S], [T])
+    assert plan["path"] == hip.hip.PATH_PREFILL and pc.instantiation(plan) == inst, plan
+    theta = 1e6 if hd == 128 else 500000.0
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, theta, norm=norm, capacity=S + T + 8, seed=S + T + hd)
+    if S:
+        kf, vf = (r.standard_normal((KV, S, hd), dtype=np.float32) for _ in range(2))
+        cache.fill(0, kf, vf)
+        blocks[0].fill_cache(kf, vf)
+    assert check_step(ctx, cache, blocks, r, [T], threads=16, what=name) < 1e-4
+    check_step(ctx, cache, blocks, r, [1], threads=16, what=name + ", then one row")
+    cache.close()
+    ctx.close()
 
 
 def test_batched_prefill_mixed_lengths(hip):
@@ -468,8 +489,10 @@ def test_decode_context_131072(hip):
 
 # ------------------------------------------------------------------ properties at full size
 def test_full_size_properties_prefill_8192(hip):
-    """T = 8192 (Llama-1B geometry): too slow for the scalar oracle on every row, so check
-    (a) sampled rows against the oracle run on just those rows, (b) causality, (c) GQA sharing."""
+    """T = 8192 (Llama-1B geometry), on top of the comparison of all rows with the oracle in
+    test_prefill_full_size_every_instantiation: (a) rows around tile and block edges against the
+    oracle run on just those rows, from the device's own cache contents, (b) causality, (c) GQA
+    sharing."""
     import torch
 
     H, KV, hd, T = 32, 8, 64, 8192
@@ -505,6 +528,42 @@ def test_full_size_properties_prefill_8192(hip):
     out2 = ctx.forward(cache, q, k2, v2, [T])
     ctx.sync()
     assert torch.equal(out2[:5000], out[:5000]) and not torch.equal(out2[5000:], out[5000:])
+
+
+# ------------------------------------------------------------------ RoPE.apply (rope.cr:7-33)
+def test_rope_apply_reference_known_answers(hip):
+    # spec/rope_kv_cache_spec.cr:5-26
+    m = np.arange(1, 9, dtype=np.float32).reshape(1, 8)
+    assert np.abs(hip.RoPE.apply(m, 0, 10000.0) - m).max() < 1e-5
+    m = np.array([[1.0, 0.0, 0.0, 0.0]], np.float32)
+    out = hip.RoPE.apply(m, 1, 10000.0)
+    assert abs(out[0, 0] - np.cos(1.0)) < 1e-4 and abs(out[0, 2] - np.sin(1.0)) < 1e-4
+
+
+@pytest.mark.parametrize("T,hd,start,theta", [(1, 8, 0, 1e4), (33, 64, 5, 1e4), (700, 128, 32000, 1e6), (9, 7, 3, 5e5),
+                                              (4, 1, 2, 1e4), (50, 33, 100, 1e4)])
+def test_rope_apply_matches_oracle(hip, T, hd, start, theta):
+    """Against orc_rope_apply.  Both sides compute in fp64 and round once; the device's fp64 pow, cos
+    and sin may differ from the host libm's in the last bit of a double, which can move a result
+    across an fp32 rounding boundary: at most one unit in the last place, and rarely."""
+    import torch
+
+    r = np.random.default_rng(T + hd)
+    x = r.standard_normal((T, hd)).astype(np.float32)
+    want = orc.rope_apply(x, start, theta)
+    got = hip.RoPE.apply(x, start, theta)
+    ulp = np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))
+    assert ulp.max() <= 1 and (ulp > 0).mean() < 1e-3, (ulp.max(), (ulp > 0).mean())
+    if hd & 1:
+        assert np.array_equal(got[:, hd - 1], x[:, hd - 1])  # the odd trailing column is copied through
+    dev = hip.RoPE.apply(torch.from_numpy(x).cuda(), start, theta)
+    torch.cuda.synchronize()
+    assert np.array_equal(dev.cpu().numpy(), got)
+    # rotation: every pair keeps its norm
+    h = hd // 2
+    n0 = x[:, :h].astype(np.float64) ** 2 + x[:, h:2 * h].astype(np.float64) ** 2
+    n1 = got[:, :h].astype(np.float64) ** 2 + got[:, h:2 * h].astype(np.float64) ** 2
+    assert np.abs(n1 - n0).max() <= 1e-5 * max(1.0, n0.max())
 
 
 # ------------------------------------------------------------------ entry points with the reference's names
