@@ -123,12 +123,24 @@ __device__ __forceinline__ int workgroup_of_tile(int t, int tiles_per_wg, const 
 // One segment of a workgroup's span: tiles [tile0, tile1) of one (sequence, kv head) pair.
 struct Segment {
   int s, kvh, R, L, n_s, tile0, tile1, token;  // R new rows; L keys visible to the last of them
+  int rot;  // the segment's tiles are visited from tile0 + rot on, wrapping round to tile0 + rot - 1
   const float *kbase, *vbase;
 };
 
+// Where a workgroup starts within a segment.  Workgroups that all walk their spans from the first
+// tile on move through memory in step, a fixed number of bytes apart, and for some distances
+// (129 or 145 tiles of 8 KiB, for one) their requests pile up on a few memory channels: a plain
+// read kernel laid out that way drops from 6.1 to 5.2 and 4.8 TB/s, and keeps 6.0 TB/s at every
+// distance when each workgroup starts at a different place of its range.  The order of the keys
+// does not matter to an online softmax.
+__device__ __forceinline__ int segment_rotation(int n_tiles, unsigned rotate) {
+  if (!rotate || n_tiles < 2) return 0;
+  return (int)(((blockIdx.x * 2654435761u) >> 12) % min((unsigned)n_tiles, rotate));
+}
+
 // The segment that starts at tile t of the stream; s: a sequence at or before t's, moved up to it.
 __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const SeqTable &st, const Shape &sh, int hd,
-                                              const float *kc, const float *vc) {
+                                              const float *kc, const float *vc, unsigned rotate) {
   while (s + 1 < st.n_seqs && t >= st.work_off[s + 1]) ++s;
   Segment g;
   g.s = s;
@@ -139,6 +151,7 @@ __device__ __forceinline__ Segment segment_at(int t, int t_end, int &s, const Se
   g.kvh = rel / g.n_s;
   g.tile0 = rel - g.kvh * g.n_s;
   g.tile1 = g.tile0 + min(g.n_s - g.tile0, t_end - t);
+  g.rot = __builtin_amdgcn_readfirstlane(segment_rotation(g.tile1 - g.tile0, rotate));
   const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)g.kvh * sh.cap * hd;
   g.kbase = kc + head_base;
   g.vbase = vc + head_base;
@@ -158,7 +171,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
     int spin_limit, int *error, SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, int pstride,
-    float c) {
+    float c, unsigned rotate) {
   using C = DecodeCfg<HD>;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
@@ -183,7 +196,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   // along them with dependent scalar loads took 2.5 us for a workgroup in the middle of 16
   // sequences).
   int s = (int)__popcll(__ballot(lane + 1 < st.n_seqs && t_begin >= st.work_off[lane + 1 < kMaxSeqs ? lane + 1 : kMaxSeqs]));
-  Segment seg = segment_at(t, t_end, s, st, sh, HD, kc, vc);
+  Segment seg = segment_at(t, t_end, s, st, sh, HD, kc, vc, rotate);
 
   f32x4 v_next[4][C::NVU];
   float qr[HD / 4];
@@ -207,16 +220,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   int par = 0;
   // The tiles of the span go to the wavefronts round-robin as one sequence, whatever segments
   // they fall into (a fresh start per segment would leave one wavefront with a tile more than
-  // its share in every segment): the first tile of the segment at stream position ts for
-  // this wavefront.
-  auto first_tile = [&](const Segment &sg, int ts) { return sg.tile0 + ((wave - (ts - t_begin)) & (NW - 1)); };
+  // its share in every segment): this wavefront's first place in the visiting order of the
+  // segment at stream position ts, and the tile at place i of that order.
+  auto first_place = [&](int ts) { return (wave - (ts - t_begin)) & (NW - 1); };
+  auto tile_at = [&](const Segment &sg, int i) {
+    const int n = sg.tile1 - sg.tile0, k = i + sg.rot;
+    return sg.tile0 + (k < n ? k : k - n);
+  };
   static_assert((NW & (NW - 1)) == 0, "round-robin by masking");
   // start fetching the tile at key row `row` into buffer `which`
   auto fetch = [&](int which, const float *kb_, const float *vb_, int row, int last_row) {
     issue_k_tile<HD>(kb_, row, last_row, my_lds + which * C::TILE_BYTES, lane);
     load_v_tile<HD>(vb_, row, last_row, col, j, v_next);
   };
-  if (first_tile(seg, t) < seg.tile1) fetch(0, seg.kbase, seg.vbase, first_tile(seg, t) * 16, seg.L - 1);
+  if (first_place(t) < seg.tile1 - seg.tile0) fetch(0, seg.kbase, seg.vbase, tile_at(seg, first_place(t)) * 16, seg.L - 1);
   load_q(seg);
 
   // the pair whose last segment this workgroup holds without holding all of it: merged at the
@@ -243,20 +260,22 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const int t_next = t + (tile1 - seg.tile0);
     const bool more = t_next < t_end;
     Segment nseg = seg;
-    if (more) nseg = segment_at(t_next, t_end, s, st, sh, HD, kc, vc);
-    const int ntile = first_tile(nseg, t_next);
-    const bool nhave = more && ntile < nseg.tile1;
+    if (more) nseg = segment_at(t_next, t_end, s, st, sh, HD, kc, vc, rotate);
+    const int nplace = first_place(t_next);
+    const bool nhave = more && nplace < nseg.tile1 - nseg.tile0;
+    const int ntile = nhave ? tile_at(nseg, nplace) : 0;
+    const int n_here = tile1 - seg.tile0;
 
     float m = -INFINITY, l = 0.f;
     f32x4 o[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    int tile = first_tile(seg, t);
+    int place = first_place(t);
     // no tile of this segment for this wavefront: on to the next one's
-    if (tile >= tile1 && nhave) fetch(par, nseg.kbase, nseg.vbase, ntile * 16, nseg.L - 1);
-    for (; tile < tile1; tile += NW) {
-      const int kb = tile * 16;
+    if (place >= n_here && nhave) fetch(par, nseg.kbase, nseg.vbase, ntile * 16, nseg.L - 1);
+    for (; place < n_here; place += NW) {
+      const int kb = tile_at(seg, place) * 16;
       const char *buf = my_lds + par * C::TILE_BYTES;
       par ^= 1;
       // everything issued so far (this tile's K copy and V loads) has landed:
@@ -270,8 +289,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       for (int r = 0; r < 4; ++r)
 #pragma unroll
         for (int u = 0; u < C::NVU; ++u) v_cur[r][u] = v_next[r][u];
-      if (tile + NW < tile1)
-        fetch(par, kbase, vbase, kb + 16 * NW, L - 1);
+      if (place + NW < n_here)
+        fetch(par, kbase, vbase, tile_at(seg, place + NW) * 16, L - 1);
       else if (nhave)
         fetch(par, nseg.kbase, nseg.vbase, ntile * 16, nseg.L - 1);
 
@@ -561,16 +580,19 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   // before / after (nullable) receive the kernel's own first and last clock reading, not the
   // time at which the stream reached them: what is between two kernels stays out
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
+  // SHAINET_HIP_DECODE_NO_ROTATE: every workgroup walks its segments from their first tile (for comparison)
+  static const unsigned rotate = getenv("SHAINET_HIP_DECODE_NO_ROTATE") ? 0u : getenv("SHAINET_HIP_DECODE_ROTATE") ? (unsigned)atoi(getenv("SHAINET_HIP_DECODE_ROTATE")) : 0x7fffffffu;
+  const size_t pad = 0;
   if (sh.hd == 64)
-    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<64, kDecodeWaves>), grid, block, 0, stream, before, after, d.q_rot,
+    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<64, kDecodeWaves>), grid, block, pad, stream, before, after, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
-                          p.n_slots, p.cols, c);
+                          p.n_slots, p.cols, c, rotate);
   else
-    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<128, kDecodeWaves>), grid, block, 0, stream, before, after, d.q_rot,
+    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<128, kDecodeWaves>), grid, block, pad, stream, before, after, d.q_rot,
                           d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
                           p.total_tiles,
-                          p.n_slots, p.cols, c);
+                          p.n_slots, p.cols, c, rotate);
   hipError_t e = hipGetLastError();
   return e;
 }

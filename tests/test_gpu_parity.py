@@ -563,7 +563,8 @@ def test_rope_apply_matches_oracle(hip, T, hd, start, theta):
     h = hd // 2
     n0 = x[:, :h].astype(np.float64) ** 2 + x[:, h:2 * h].astype(np.float64) ** 2
     n1 = got[:, :h].astype(np.float64) ** 2 + got[:, h:2 * h].astype(np.float64) ** 2
-    assert np.abs(n1 - n0).max() <= 1e-5 * max(1.0, n0.max())
+    if h:
+        assert np.abs(n1 - n0).max() <= 1e-5 * max(1.0, n0.max())
 
 
 # ------------------------------------------------------------------ entry points with the reference's names
