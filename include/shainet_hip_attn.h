@@ -151,6 +151,24 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
                          const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                          float *out, int mem);
 
+/* shainet_attn_forward for decode calls, for callers that cannot allocate device memory while they
+ * call it (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * this variant allocates nothing.  It has no counterpart in the reference.  Device pointers only,
+ * asynchronous on the context's stream, same results as shainet_attn_forward.  What that call
+ * grows on demand comes from a fixed array in device memory instead (8.06 MiB per GPU, held until
+ * the process ends): 2 MiB for the rotated query rows (sum new_tokens x num_heads x head_dim
+ * <= 524288 floats), 6 MiB for the split's partial results and 32 KiB of flag words (with the
+ * default 256 workgroups: any batch of up to 64 sequences of head_dim <= 128).  Limits, each
+ * refused with SHAINET_HIP_ERR_ARGUMENT or SHAINET_HIP_ERR_CAPACITY and a message, nothing
+ * appended: head_dim 64 or 128; at most 32 / (num_heads / num_kv_heads) new rows per sequence
+ * (the calls the split-K decode kernel takes); every position below the max_positions the
+ * context was created with; sizes within the array.  All calls on one GPU share the array:
+ * two calls of this entry point that overlap in time on one GPU (different contexts on
+ * different streams) race; calls on one context, or one after the other, do not. */
+int shainet_attn_forward_noalloc(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const int *seq_ids,
+                                 const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
+                                 float *out);
+
 /* Copy of the rotated query rows of the last shainet_attn_forward call
  * ([sum new_tokens, num_heads*head_dim], host): lets a test check RoPE positions
  * and QK-norm of Q exactly (llama_block.cr:332-344). */

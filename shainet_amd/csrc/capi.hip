@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -212,13 +213,31 @@ int ensure_decode_flags(shainet_attn_ctx *c, size_t n, hipStream_t stream) {
   return SHAINET_HIP_OK;
 }
 
+// Device memory a forward call's kernels use beyond its inputs and outputs, when the caller of
+// run_attention brings it along instead of letting the context allocate it on demand.
+struct Workspace {
+  float *q_rot;
+  size_t q_rot_floats;
+  float *partials;
+  size_t partial_floats;
+  unsigned *flags;  // zero at launch
+  size_t flag_words;
+  unsigned *lost_marks;  // flag_words words: where the test of the give-up path sends the marks
+};
+
 // Attention over a cache: shared by the fused entry point and by attention_kv_f32.
 // prep != nullptr: the rows are raw projection outputs; the prep kernel does bias,
 // QK-norm, RoPE and the append first.  prep == nullptr: q_rot holds rotated
 // queries and the cache already holds the new rows.
+// ws != nullptr: nothing is allocated; the split-K decode path only.
 int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc, float *out, SeqTable &st,
-                  const Shape &sh, int total_tokens, float scale, hipStream_t stream, const PrepArgs *prep) {
+                  const Shape &sh, int total_tokens, float scale, hipStream_t stream, const PrepArgs *prep,
+                  const Workspace *ws = nullptr) {
   const Path path = choose_path(st, sh);
+  if (ws && path != Path::kDecodeSplitK)
+    return fail(SHAINET_HIP_ERR_ARGUMENT,
+                "the entry point that allocates nothing takes decode calls only: at most %d new rows per sequence "
+                "with this head geometry (head_dim 64 or 128)", 32 / (sh.g < 1 ? 1 : sh.g));
   // the MFMA prefill kernels address the rows of a (sequence, kv head) by a 32-bit byte offset;
   // said before anything is written to the cache
   if (path == Path::kPrefillMfma && (long long)sh.cap * sh.hd * 4 > 0xffffffffLL)
@@ -227,7 +246,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
                 sh.cap, sh.hd);
   hipError_t e;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  if (c->profiling) {
+  if (c->profiling && !ws) {
     if (hipEventCreate(&ev0) != hipSuccess || hipEventCreate(&ev1) != hipSuccess)
       return fail(SHAINET_HIP_ERR_RUNTIME, "hipEventCreate failed");
     c->prof_events.push_back(ev0);
@@ -237,18 +256,29 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     SeqTable att;  // the attention kernel's view: long runs of new rows as two entries
     if (!decode_entries(st, sh, att)) return fail(SHAINET_HIP_ERR_RUNTIME, "decode entries do not fit");
     const DecodePlan plan = plan_decode(att, sh, c->decode_wgs_override);
-    int rc = c->partials.reserve(decode_partial_floats(sh, plan));
-    if (!rc) rc = ensure_decode_flags(c, decode_flag_words(plan), stream);
-    if (rc) return rc;
     DecodeArgs d;
+    if (ws) {
+      if (decode_partial_floats(sh, plan) > ws->partial_floats || decode_flag_words(plan) > ws->flag_words)
+        return fail(SHAINET_HIP_ERR_CAPACITY,
+                    "this call needs %zu floats of partial results and %zu flag words; the static scratch holds "
+                    "%zu and %zu", decode_partial_floats(sh, plan), decode_flag_words(plan), ws->partial_floats,
+                    ws->flag_words);
+      d.partials = ws->partials;
+      d.part_flag = ws->flags;
+      d.flag_set = c->test_lose_marks ? ws->lost_marks : nullptr;
+    } else {
+      int rc = c->partials.reserve(decode_partial_floats(sh, plan));
+      if (!rc) rc = ensure_decode_flags(c, decode_flag_words(plan), stream);
+      if (rc) return rc;
+      d.partials = c->partials.p;
+      d.part_flag = c->part_flag;
+      d.flag_set = c->test_lose_marks ? c->part_flag + c->part_flag_cap : nullptr;
+    }
     d.q_rot = q_rot;
     d.kc = kc;
     d.vc = vc;
     d.out = out;
-    d.partials = c->partials.p;
-    d.part_flag = c->part_flag;
     d.error = c->error;
-    d.flag_set = c->test_lose_marks ? c->part_flag + c->part_flag_cap : nullptr;
     d.spin_limit = c->test_lose_marks ? 2000 : 0;
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);
@@ -590,10 +620,29 @@ int shainet_attn_forward(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *s
 
 // The same with the rows of q, k and v at given strides (device pointers): lets a
 // caller hand over the three column blocks of one fused projection output.
+namespace {
+int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, const int *new_tokens, int n_seqs,
+                 const float *q, const float *k, const float *v, long long q_stride, long long k_stride,
+                 long long v_stride, float *out, int mem, const Workspace *ws);
+}
+
 int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids,
                                  const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                                  long long q_stride, long long k_stride, long long v_stride, float *out, int mem) {
+  return forward_core(c, kc, seq_ids, new_tokens, n_seqs, q, k, v, q_stride, k_stride, v_stride, out, mem, nullptr);
+}
+
+namespace {
+
+// ws != nullptr: device pointers only, and nothing is allocated: what the context would grow on
+// demand (cos/sin table, rotated-query rows, split-K partials and their flags) must already be
+// large enough or come with ws.
+int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, const int *new_tokens, int n_seqs,
+                 const float *q, const float *k, const float *v, long long q_stride, long long k_stride,
+                 long long v_stride, float *out, int mem, const Workspace *ws) {
   if (!c || !kc || kc->ctx != c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (ws && mem != SHAINET_HIP_MEM_DEVICE)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "the entry point that allocates nothing takes device pointers only");
   if (!new_tokens || !q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (n_seqs < 1 || n_seqs > SHAINET_HIP_MAX_BATCH)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", SHAINET_HIP_MAX_BATCH);
@@ -626,9 +675,23 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   st.tok_off[n_seqs] = (int)total;
   const int rows = (int)total;
   const size_t q_floats = (size_t)rows * c->H * c->hd, kv_floats = (size_t)rows * c->KV * c->hd;
-  int rc = ensure_rope_table(c, max_pos);
-  if (!rc) rc = c->q_rot.reserve(q_floats);
-  if (rc) return rc;
+  int rc = SHAINET_HIP_OK;
+  float *q_rot = nullptr;
+  if (ws) {
+    if (max_pos > c->rope_positions)
+      return fail(SHAINET_HIP_ERR_CAPACITY,
+                  "position %d is beyond the %d positions of the context's cos/sin table: create the context "
+                  "with max_positions of at least the cache capacity", max_pos - 1, c->rope_positions);
+    if (q_floats > ws->q_rot_floats)
+      return fail(SHAINET_HIP_ERR_CAPACITY, "%d rows of %d query floats exceed the %zu floats of static scratch "
+                  "for rotated queries", rows, c->H * c->hd, ws->q_rot_floats);
+    q_rot = ws->q_rot;
+  } else {
+    rc = ensure_rope_table(c, max_pos);
+    if (!rc) rc = c->q_rot.reserve(q_floats);
+    if (rc) return rc;
+    q_rot = c->q_rot.p;
+  }
 
   const float *dq = q, *dk = k, *dv = v;
   float *dout = out;
@@ -662,20 +725,85 @@ int shainet_attn_forward_strided(shainet_attn_ctx *c, shainet_kv_cache *kc, cons
   pa.k_norm = c->d_k_norm;
   pa.eps = c->eps;
   pa.rope_tab = c->d_rope;
-  pa.q_rot = c->q_rot.p;
+  pa.q_rot = q_rot;
   pa.kc = kc->k;
   pa.vc = kc->v;
-  rc = run_attention(c, c->q_rot.p, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa);
+  rc = run_attention(c, q_rot, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa, ws);
   if (rc) return rc;  // the cached lengths stay as they were: the call did not happen
   // the rows are in the cache once this call's kernels have run: @cache_len = total_len (llama_block.cr:288-289)
   for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
-  c->last_rows = rows;
+  c->last_rows = ws ? 0 : rows;  // shainet_attn_last_q_rot reads the context's own buffer
   if (mem == SHAINET_HIP_MEM_HOST) {
     HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     return check_error_word(c->error);
   }
   return SHAINET_HIP_OK;
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------
+//
+// Static device memory for what shainet_attn_forward's decode path otherwise allocates on demand:
+// the flag words of the split (zero at launch), the rotated query rows and the partial results.
+// Every GPU the library runs on holds its own copy of the array at its own address until the
+// process ends; all calls on a GPU share it, so two such calls that overlap on one GPU race.
+constexpr size_t kScratchFlagWords = 8192;              // 32 KiB of flags + 32 KiB for the give-up test's lost marks
+constexpr size_t kScratchQRotFloats = 512 * 1024;       // 2 MiB: e.g. 128 rows of 32 heads x 128
+constexpr size_t kScratchPartialFloats = 1536 * 1024;   // 6 MiB: e.g. 776 slots x 16 columns x (128 + 2)
+constexpr size_t kScratchBytes =
+    2 * kScratchFlagWords * sizeof(unsigned) + (kScratchQRotFloats + kScratchPartialFloats) * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, once asked for
+std::mutex g_scratch_lock;
+
+// The address of this device's copy of `scratch` (the array's name is a host-side stand-in, not
+// a device address: only hipGetSymbolAddress tells where the array lives on the current device).
+int scratch_on_current_device(unsigned char **out) {
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(SHAINET_HIP_ERR_RUNTIME, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(SHAINET_HIP_ERR_RUNTIME, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = (unsigned char *)g_scratch_ptr[dev];
+  return SHAINET_HIP_OK;
+}
+
+__global__ void fill_words_kernel(unsigned *p, unsigned value, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+
+}  // namespace
+
+extern "C" int shainet_attn_forward_noalloc(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids,
+                                            const int *new_tokens, int n_seqs, const float *q, const float *k,
+                                            const float *v, float *out) {
+  if (!c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  unsigned char *base = nullptr;
+  if (int rc = scratch_on_current_device(&base)) return rc;
+  Workspace ws;
+  ws.flags = (unsigned *)base;
+  ws.flag_words = kScratchFlagWords;
+  ws.lost_marks = ws.flags + kScratchFlagWords;
+  ws.q_rot = (float *)(base + 2 * kScratchFlagWords * sizeof(unsigned));
+  ws.q_rot_floats = kScratchQRotFloats;
+  ws.partials = ws.q_rot + kScratchQRotFloats;
+  ws.partial_floats = kScratchPartialFloats;
+  // The array keeps what the last call on this GPU left in it.  The flag words must be zero at
+  // launch; a launch leaves them so unless a wait was given up, so they are cleared every time, with
+  // a fill kernel (a caller may be capturing the stream into a graph, where memset nodes are unsafe).
+  hipLaunchKernelGGL(fill_words_kernel, dim3((unsigned)((kScratchFlagWords + 255) / 256)), dim3(256), 0, c->stream,
+                     ws.flags, 0u, kScratchFlagWords);
+  HIP_TRY(hipGetLastError());
+  return forward_core(c, kc, seq_ids, new_tokens, n_seqs, q, k, v, (long long)c->H * c->hd, (long long)c->KV * c->hd,
+                      (long long)c->KV * c->hd, out, SHAINET_HIP_MEM_DEVICE, &ws);
 }
 
 // The owner of a context (a block, a model) makes the context's kernels report into the owner's

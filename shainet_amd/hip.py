@@ -72,6 +72,8 @@ _SIGNATURES = {
     "shainet_kv_cache_read": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p]),
     "shainet_attn_forward": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
                                        C.c_void_p, C.c_void_p, C.c_int]),
+    "shainet_attn_forward_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
+                                               C.c_void_p, C.c_void_p]),
     "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
     "shainet_attn_describe_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _i32p, _i32p, _i32p]),
     "shainet_rope_apply": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_double, C.c_int]),
@@ -375,6 +377,23 @@ class AttnContext:
         _check(lib().shainet_attn_forward(self._h, cache._h, ids, nt, n, _ptr(q), _ptr(k), _ptr(v), _ptr(out), mem))
         return out
 
+
+    def forward_noalloc(self, cache, q, k, v, new_tokens, seq_ids=None, out=None):
+        """shainet_attn_forward_noalloc: decode calls on torch CUDA tensors, with every buffer the
+        kernels need beyond inputs and outputs taken from the library's static device array."""
+        n = len(new_tokens)
+        nt = (C.c_int * n)(*new_tokens)
+        ids = (C.c_int * n)(*seq_ids) if seq_ids is not None else None
+        rows = sum(new_tokens)
+        assert q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        assert tuple(q.shape) == (rows, self.q_dim) and tuple(k.shape) == (rows, self.kv_dim)
+        assert tuple(v.shape) == tuple(k.shape)
+        if out is None:
+            import torch
+
+            out = torch.empty_like(q)
+        _check(lib().shainet_attn_forward_noalloc(self._h, cache._h, ids, nt, n, _ptr(q), _ptr(k), _ptr(v), _ptr(out)))
+        return out
 
     def prepared(self, cache, q, k, v, new_tokens, out, seq_ids=None):
         """A zero-argument callable that repeats this device-pointer forward call with nothing but
