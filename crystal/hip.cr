@@ -50,7 +50,8 @@ module SHAInet
       @@kernels_handle
     end
 
-    private def sym(name : String) : Pointer(Void)
+    # Address of an entry point of the kernel library (also used by hip_model.cr).
+    def sym(name : String) : Pointer(Void)
       h = kernels_handle
       raise "HIP kernels not available" if h.null?
       s = LibC.dlsym(h, name)
@@ -141,7 +142,7 @@ module SHAInet
     # ---- fused entry points (include/shainet_hip_attn.h) ----------------------
     alias Handle = Pointer(Void)
 
-    private def check(status : Int32)
+    def check(status : Int32)
       return if status == 0
       msg = last_error
       raise ArgumentError.new(msg) if status == 1
@@ -217,6 +218,34 @@ module SHAInet
         status = fn.call(cache, capacity)
       end
       check(status)
+    end
+
+    # RoPE.apply (src/shainet/transformer/rope.cr:7-33) on host rows: [seq_len, head_dim] in and out.
+    def rope_apply(x : Pointer(Float32), out_ptr : Pointer(Float32), seq_len : Int32, head_dim : Int32,
+                   start_pos : Int32, theta : Float64)
+      fn = Proc(Pointer(Float32), Pointer(Float32), Int32, Int32, Int32, Float64, Int32, Int32).new(sym("shainet_rope_apply"), Pointer(Void).null)
+      check fn.call(x, out_ptr, seq_len, head_dim, start_pos, theta, MEM_HOST)
+    end
+
+    # y[rows, n] = x[rows, k] W[k, n] (+ res) on device pointers: what LlamaBlock#gpu_matmul dispatches
+    # (llama_block.cr:726-768); stream null = the default stream.
+    def matmul_f32(x : Pointer(Float32), x_stride : Int64, w : Pointer(Float32), res : Pointer(Float32),
+                   y : Pointer(Float32), rows : Int32, k : Int32, n : Int32, stream : Pointer(Void) = Pointer(Void).null)
+      fn = Proc(Pointer(Float32), Int64, Pointer(Float32), Pointer(Float32), Pointer(Float32), Int32, Int32, Int32, Pointer(Void), Int32).new(sym("shainet_hip_matmul_f32"), Pointer(Void).null)
+      check fn.call(x, x_stride, w, res, y, rows, k, n, stream)
+    end
+
+    # Decode calls on device pointers that allocate nothing (graph capture, tight serving loops):
+    # shainet_attn_forward_noalloc.  One sequence (cache slot 0), new_tokens rows.
+    def attn_forward_noalloc(ctx : Handle, cache : Handle, new_tokens : Int32,
+                             q : Pointer(Float32), k : Pointer(Float32), v : Pointer(Float32), out_ptr : Pointer(Float32))
+      fn = Proc(Handle, Handle, Pointer(Int32), Pointer(Int32), Int32, Pointer(Float32), Pointer(Float32), Pointer(Float32), Pointer(Float32), Int32).new(sym("shainet_attn_forward_noalloc"), Pointer(Void).null)
+      nt = new_tokens
+      check fn.call(ctx, cache, Pointer(Int32).null, pointerof(nt), 1, q, k, v, out_ptr)
+    end
+
+    def attn_sync(ctx : Handle)
+      check Proc(Handle, Int32).new(sym("shainet_attn_sync"), Pointer(Void).null).call(ctx)
     end
 
     # Host-pointer mode: q, k, v and out are SimpleMatrix buffers; returns with out filled.

@@ -1,62 +1,63 @@
 # Crystal binding of the layer- and model-level entry points of
 # libshainet_hip_kernels.so: the whole LlamaBlock, the model walk of Network#run,
-# the Sampler's device half and HFLoader.load_llama.  The library is linked
-# directly (`@[Link]`), the way the reference links its runtime library
-# (cuda.cr:9-19); every function returns the Int32 status of the rest of the
-# library (0 = ok, 1 = ArgumentError, 3 = allocation failed).
+# the Sampler's device half and HFLoader.load_llama.  Bound like the rest of the
+# kernel library, by dlopen / dlsym (hip.cr: `HIP.sym`, the idiom of cuda.cr:841-852),
+# so that a build that never opens the library still links; every function returns
+# the Int32 status of the rest of the library (0 = ok, 1 = ArgumentError,
+# 3 = allocation failed).
 #
 # Written without a Crystal compiler at hand (none exists in the build image).
 require "./hip"
 
 module SHAInet
   module HIP
-    @[Link("shainet_hip_kernels")]
-    lib LibModel
-      type Attn = Void*
-      type Block = Void*
-      type Model = Void*
+    alias Model = Pointer(Void)
+    alias Block = Pointer(Void)
 
-      fun shainet_hip_last_error : LibC::Char*
+    # One cached Proc per entry point: `model_fn(name, arg types..., return type)`.
+    macro model_fn(name, *types)
+      @@{{name.id}}_proc : Proc({{types.splat}})?
 
-      fun shainet_llama_block_create(out : Block*, d_model : Int32, num_heads : Int32, ff_hidden : Int32, eps : Float64,
-                                     rope_theta : Float64, num_kv_heads : Int32, head_dim : Int32) : Int32
-      fun shainet_llama_block_destroy(block : Block) : Int32
-      fun shainet_llama_block_attn(block : Block) : Attn
-      fun shainet_llama_block_set_norms(block : Block, norm1 : Float32*, norm2 : Float32*) : Int32
-      fun shainet_llama_block_set_ffn(block : Block, gate : Float32*, up : Float32*, down : Float32*) : Int32
-      fun shainet_llama_block_clear_cache(block : Block) : Int32
-      fun shainet_llama_block_cache_len(block : Block) : Int32
-      fun shainet_llama_block_forward_cached(block : Block, x : Float32*, new_tokens : Int32, out : Float32*, mem : Int32) : Int32
+      def self.{{name.id}}(*args)
+        fn = (@@{{name.id}}_proc ||= Proc({{types.splat}}).new(HIP.sym({{name.id.stringify}}), Pointer(Void).null))
+        fn.call(*args)
+      end
+    end
 
-      fun shainet_llama_attn_set_rope(attn : Attn, rope_theta : Float64, rope_freqs : Float32*) : Int32
-      fun shainet_llama_attn_set_qk_norm(attn : Attn, q_norm : Float32*, q_len : Int32, k_norm : Float32*, k_len : Int32) : Int32
-      fun shainet_llama_attn_set_bias(attn : Attn, b_q : Float32*, q_len : Int32, b_k : Float32*, k_len : Int32,
-                                      b_v : Float32*, v_len : Int32) : Int32
-      fun shainet_llama_attn_set_weights(attn : Attn, w_q : Float32*, w_k : Float32*, w_v : Float32*, w_o : Float32*) : Int32
+    module LibModel
+      HIP.model_fn shainet_llama_block_create, Pointer(Block), Int32, Int32, Int32, Float64, Float64, Int32, Int32, Int32
+      HIP.model_fn shainet_llama_block_destroy, Block, Int32
+      HIP.model_fn shainet_llama_block_attn, Block, Pointer(Void)
+      HIP.model_fn shainet_llama_block_set_norms, Block, Pointer(Float32), Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_block_set_ffn, Block, Pointer(Float32), Pointer(Float32), Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_block_clear_cache, Block, Int32
+      HIP.model_fn shainet_llama_block_cache_len, Block, Int32
+      HIP.model_fn shainet_llama_block_forward_cached, Block, Pointer(Float32), Int32, Pointer(Float32), Int32, Int32
+      HIP.model_fn shainet_llama_block_forward, Block, Pointer(Float32), Int32, Pointer(Float32), Int32, Int32
 
-      fun shainet_llama_model_create(out : Model*, vocab : Int32, d_model : Int32, n_layers : Int32, num_heads : Int32,
-                                     num_kv_heads : Int32, head_dim : Int32, ff_hidden : Int32, eps : Float64,
-                                     rope_theta : Float64) : Int32
-      fun shainet_llama_model_destroy(model : Model) : Int32
-      fun shainet_llama_model_block(model : Model, layer : Int32) : Block
-      fun shainet_llama_model_set_embedding(model : Model, table : Float32*) : Int32
-      fun shainet_llama_model_set_final_norm(model : Model, gamma : Float32*) : Int32
-      fun shainet_llama_model_set_lm_head(model : Model, weights : Float32*, bias : Float32*) : Int32
-      fun shainet_llama_model_clear_cache(model : Model) : Int32
-      fun shainet_llama_model_run(model : Model, tokens : Int32*, n_tokens : Int32, logits : Float32*) : Int32
-      fun shainet_llama_model_greedy(model : Model, token : Int32*) : Int32
-      fun shainet_llama_model_repetition_penalty(model : Model, recent_ids : Int32*, n : Int32, penalty : Float64) : Int32
-      fun shainet_llama_model_topk(model : Model, k : Int32, ids : Int32*, vals : Float32*, count : Int32*) : Int32
-      fun shainet_llama_model_generate_greedy(model : Model, max_tokens : Int32, stop_ids : Int32*, n_stop : Int32,
-                                              out : Int32*, n_out : Int32*) : Int32
-      fun shainet_hf_load_llama(model_dir : LibC::Char*, out : Model*) : Int32
+      HIP.model_fn shainet_llama_attn_set_rope, Pointer(Void), Float64, Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_attn_set_qk_norm, Pointer(Void), Pointer(Float32), Int32, Pointer(Float32), Int32, Int32
+      HIP.model_fn shainet_llama_attn_set_bias, Pointer(Void), Pointer(Float32), Int32, Pointer(Float32), Int32, Pointer(Float32), Int32, Int32
+      HIP.model_fn shainet_llama_attn_set_weights, Pointer(Void), Pointer(Float32), Pointer(Float32), Pointer(Float32), Pointer(Float32), Int32
+
+      HIP.model_fn shainet_llama_model_create, Pointer(Model), Int32, Int32, Int32, Int32, Int32, Int32, Int32, Float64, Float64, Int32
+      HIP.model_fn shainet_llama_model_destroy, Model, Int32
+      HIP.model_fn shainet_llama_model_block, Model, Int32, Block
+      HIP.model_fn shainet_llama_model_set_embedding, Model, Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_model_set_final_norm, Model, Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_model_set_lm_head, Model, Pointer(Float32), Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_model_clear_cache, Model, Int32
+      HIP.model_fn shainet_llama_model_run, Model, Pointer(Int32), Int32, Pointer(Float32), Int32
+      HIP.model_fn shainet_llama_model_greedy, Model, Pointer(Int32), Int32
+      HIP.model_fn shainet_llama_model_repetition_penalty, Model, Pointer(Int32), Int32, Float64, Int32
+      HIP.model_fn shainet_llama_model_topk, Model, Int32, Pointer(Int32), Pointer(Float32), Pointer(Int32), Int32
+      HIP.model_fn shainet_llama_model_sample, Model, Int32, Float64, Float64, Pointer(Int32), Int32
+      HIP.model_fn shainet_llama_model_generate_greedy, Model, Int32, Pointer(Int32), Int32, Pointer(Int32), Pointer(Int32), Int32
+      HIP.model_fn shainet_hf_load_llama, Pointer(UInt8), Pointer(Model), Int32
     end
 
     def self.check!(status : Int32)
-      return if status == 0
-      msg = String.new(LibModel.shainet_hip_last_error)
-      raise ArgumentError.new(msg) if status == 1
-      raise msg
+      HIP.check(status)
     end
 
     # Network#run(ids) with use_kv_cache for a network whose LLaMA stack lives on the
@@ -64,13 +65,13 @@ module SHAInet
     class DeviceLlama
       getter vocab : Int32
 
-      def initialize(@handle : LibModel::Model, @vocab : Int32)
+      def initialize(@handle : Model, @vocab : Int32)
       end
 
       # HFLoader.load_llama(model_dir) (hf_loader.cr:277-412), dense models
       def self.load(model_dir : String, vocab : Int32) : DeviceLlama
-        h = Pointer(Void).null.as(LibModel::Model)
-        HIP.check!(LibModel.shainet_hf_load_llama(model_dir, pointerof(h)))
+        h = Model.null
+        HIP.check!(LibModel.shainet_hf_load_llama(model_dir.to_unsafe, pointerof(h)))
         new(h, vocab)
       end
 
@@ -88,6 +89,15 @@ module SHAInet
       def greedy : Int32
         id = 0
         HIP.check!(LibModel.shainet_llama_model_greedy(@handle, pointerof(id)))
+        id
+      end
+
+      # Sampler#sample (text/sampler.cr:88-150) on the device logits: top-k, temperature softmax
+      # over the survivors and the inverse-CDF pick for the uniform draw `r` in [0, 1) that the
+      # caller's random generator made.
+      def sample(top_k : Int32, temperature : Float64, r : Float64) : Int32
+        id = 0
+        HIP.check!(LibModel.shainet_llama_model_sample(@handle, top_k, temperature, r, pointerof(id)))
         id
       end
 

@@ -228,6 +228,17 @@ int shainet_llama_attn_forward_cached(shainet_llama_attn *layer, const float *x,
  * position 0 over the seq_len rows of x alone; @cache_len and the cached rows are left as they are. */
 int shainet_llama_attn_forward_full(shainet_llama_attn *layer, const float *x, int seq_len, float *out);
 
+/* The projection product by itself: y[rows, n] = x[rows, k] W[k, n] (+ res[rows, n]), fp32, row-major,
+ * device pointers, asynchronous on `stream` (NULL = the default stream); the rows of x are
+ * x_stride floats apart, y and res are dense, res may be NULL or y.  What LlamaBlock#gpu_matmul
+ * dispatches (llama_block.cr:726-768: SimpleMatrix#* on the host, cuBLAS SGEMM on the device,
+ * cuda.cr:237-247): up to 16 rows run the split GEMV of the decode step, more rows the MFMA
+ * kernel of the prefill.  fp32 accumulation (the host path of the reference accumulates in
+ * fp64, simple_matrix.cr:61-74).  The handle-less calls share one grow-only scratch buffer:
+ * one caller at a time. */
+int shainet_hip_matmul_f32(const float *x, long long x_stride, const float *w, const float *res, float *y, int rows,
+                           int k, int n, void *stream);
+
 /* ---- the whole block ---------------------------------------------------------
  *
  * LlamaBlock#forward_cached (llama_block.cr:189-196) with a dense SwiGLU
@@ -269,7 +280,8 @@ int shainet_llama_block_forward(shainet_llama_block *block, const float *x, int 
  * last run: Sampler.greedy (text/sampler.cr:38-53), Sampler#apply_repetition_penalty!
  * (59-81) and the top-k selection of Sampler#sample (88-116); the temperature
  * softmax and the draw over the k survivors (118-150) stay with the caller, who
- * owns the random generator. */
+ * owns the random generator, or run on the device too with shainet_llama_model_sample, which
+ * takes the uniform draw as an argument. */
 typedef struct shainet_llama_model shainet_llama_model;
 int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model, int n_layers, int num_heads,
                                int num_kv_heads, int head_dim, int ff_hidden, double eps, double rope_theta);
@@ -309,6 +321,11 @@ int shainet_llama_model_repetition_penalty(shainet_llama_model *model, const int
 /* the k largest logits (1 <= k <= 256), NaN excluded, descending, equal values by ascending id;
  * *count = entries written (< k when fewer are eligible) */
 int shainet_llama_model_topk(shainet_llama_model *model, int k, int *ids, float *vals, int *count);
+/* Sampler#sample (text/sampler.cr:88-150) on the device logits, whole: the top-k selection, the softmax
+ * of v / temperature over the survivors in fp64 and the inverse-CDF pick for the uniform draw r in [0, 1)
+ * that the caller's random generator made (@rng.rand, sampler.cr:136); *token = 0 when no logit is
+ * eligible (all NaN).  top_k in [1, 256], temperature > 0 (sampler.cr:24-25: ArgumentError otherwise). */
+int shainet_llama_model_sample(shainet_llama_model *model, int top_k, double temperature, double r, int *token);
 
 /* ---- SafeTensors and the HuggingFace loader --------------------------------------
  *

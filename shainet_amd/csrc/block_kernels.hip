@@ -237,6 +237,33 @@ __global__ __launch_bounds__(256) void topk_merge_kernel(const float *__restrict
   }
 }
 
+// Sampler#sample after its top-k selection (text/sampler.cr:118-150): the temperature softmax over
+// the survivors and the inverse-CDF pick for the uniform draw r, one lane, in the reference's order
+// and number types (fp64 throughout).  ids / vals: the selection, descending; *count entries.
+__global__ void sample_pick_kernel(const int *__restrict__ ids, const float *__restrict__ vals,
+                                   const int *__restrict__ count, double temperature, double r, int *__restrict__ out) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const int n = *count;
+  if (n <= 0) {  // all-NaN row: nothing to sample (sampler.cr:121)
+    *out = 0;
+    return;
+  }
+  const double max_val = (double)vals[0] / temperature;  // descending order: element 0 is the maximum
+  double sum = 0.0;
+  for (int i = 0; i < n; ++i) sum += exp((double)vals[i] / temperature - max_val);
+  const double inv_sum = 1.0 / sum;
+  double cumulative = 0.0;
+  int best = ids[n - 1];
+  for (int i = 0; i < n; ++i) {
+    cumulative += exp((double)vals[i] / temperature - max_val) * inv_sum;
+    if (r <= cumulative) {
+      best = ids[i];
+      break;
+    }
+  }
+  *out = best;
+}
+
 // RoPE.apply (rope.cr:7-33): one lane per (row, pair).  Everything in fp64 as the reference has
 // it (Float32 operands widened, `theta ** (2.0 * i / head_dim)`, the angle, Math.cos / Math.sin,
 // both products and their difference or sum), rounded once when the result is stored.
@@ -313,6 +340,13 @@ hipError_t launch_rope_apply(const float *x, float *out, int seq_len, int head_d
   if ((items + 255) / 256 > 0x7fffffffLL) return hipErrorInvalidValue;
   hipLaunchKernelGGL(rope_apply_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, x, out, seq_len,
                      head_dim, start_pos, theta);
+  return hipGetLastError();
+}
+
+hipError_t launch_sample_pick(const int *ids, const float *vals, const int *count, double temperature, double r,
+                              int *out, hipStream_t stream) {
+  if (!ids || !vals || !count || !out || !(temperature > 0.0)) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(sample_pick_kernel, dim3(1), dim3(64), 0, stream, ids, vals, count, temperature, r, out);
   return hipGetLastError();
 }
 

@@ -40,4 +40,10 @@ size_t topk_scratch_bytes(int vocab, int k);
 hipError_t launch_topk(const float *logits, int vocab, int k, bool finite_only, void *scratch, int *out_ids,
                        float *out_vals, int *out_count, hipStream_t stream, int fallback_id = -1);
 
+// The rest of Sampler#sample (text/sampler.cr:118-150) on a selection launch_topk made: softmax of
+// vals / temperature over the *count survivors and the pick for the uniform draw r in [0, 1);
+// *out = the chosen id (0 when nothing was eligible).
+hipError_t launch_sample_pick(const int *ids, const float *vals, const int *count, double temperature, double r,
+                              int *out, hipStream_t stream);
+
 }  // namespace shainet

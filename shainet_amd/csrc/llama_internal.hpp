@@ -60,14 +60,10 @@ struct Fused {
 
 // y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows
 // (decode) run as one hand-written split GEMV with the norm and the epilogue
-// inside; more rows run as a library SGEMM (rocBLAS or hipBLASLt by shape, the
-// counterpart of the reference's cuBLAS SGEMM, cuda.cr:237-247) between the separate
-// norm and epilogue kernels.
-struct LtState;
+// inside; more rows run as the MFMA product of gemm_kernel.hip (the counterpart of
+// the reference's cuBLAS SGEMM, cuda.cr:237-247) after the separate norm kernel,
+// with the residual add in its epilogue and the SwiGLU activation as a kernel of its own.
 struct Projector {
-  void *blas = nullptr;
-  LtState *lt = nullptr;
-  bool lt_broken = false;
   DevF scratch, normed, wide;
   // split products: a word per partial that says when it is complete (zero between launches)
   unsigned *flags = nullptr;
@@ -80,10 +76,9 @@ struct Projector {
   void release();
 
  private:
-  int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream);
   // res != nullptr: y = res + x W
-  int gemm_lt(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
-              const float *res = nullptr);
+  int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
+           const float *res = nullptr);
 };
 
 // Replace *dst (device, hipMalloc'ed or null) by a copy of n host floats.

@@ -99,7 +99,7 @@ int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *v
     m->topk_scratch_cap = need;
   }
   if (!m->d_ids) {
-    if (hipMalloc((void **)&m->d_ids, (kMaxTopK + 1) * sizeof(int)) != hipSuccess ||
+    if (hipMalloc((void **)&m->d_ids, (kMaxTopK + 2) * sizeof(int)) != hipSuccess ||
         hipMalloc((void **)&m->d_vals, kMaxTopK * sizeof(float)) != hipSuccess)
       return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   }
@@ -347,6 +347,37 @@ int shainet_llama_model_repetition_penalty(shainet_llama_model *m, const int *re
 int shainet_llama_model_topk(shainet_llama_model *m, int k, int *ids, float *vals, int *count) {
   if (!m || !ids || !vals || !count) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   return run_topk(m, k, false, ids, vals, count);
+}
+
+int shainet_llama_model_sample(shainet_llama_model *m, int k, double temperature, double r, int *token) {
+  if (!m || !token) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (!m->have_logits) return fail(SHAINET_HIP_ERR_ARGUMENT, "no logits: call shainet_llama_model_run first");
+  if (k < 1 || k > kMaxTopK) return fail(SHAINET_HIP_ERR_ARGUMENT, "top_k must be in [1, 256]");  // sampler.cr:24
+  if (!(temperature > 0.0)) return fail(SHAINET_HIP_ERR_ARGUMENT, "temperature must be > 0");     // sampler.cr:25
+  const size_t need = topk_scratch_bytes(m->vocab, k);
+  if (need > m->topk_scratch_cap) {
+    if (m->topk_scratch) (void)hipFree(m->topk_scratch);
+    m->topk_scratch = nullptr;
+    m->topk_scratch_cap = 0;
+    if (hipMalloc(&m->topk_scratch, need) != hipSuccess) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+    m->topk_scratch_cap = need;
+  }
+  if (!m->d_ids) {
+    if (hipMalloc((void **)&m->d_ids, (kMaxTopK + 2) * sizeof(int)) != hipSuccess ||
+        hipMalloc((void **)&m->d_vals, kMaxTopK * sizeof(float)) != hipSuccess)
+      return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  }
+  // dividing by a positive temperature keeps the order of the logits: the selection over v / t
+  // (sampler.cr:100-115) is the selection over v
+  hipError_t e = launch_topk(m->logits.p, m->vocab, k, false, m->topk_scratch, m->d_ids, m->d_vals,
+                             m->d_ids + kMaxTopK, m->stream);
+  if (e == hipSuccess)
+    e = launch_sample_pick(m->d_ids, m->d_vals, m->d_ids + kMaxTopK, temperature, r, m->d_ids + kMaxTopK + 1, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("sample launch: ") + hipGetErrorString(e));
+  if (hipMemcpyAsync(token, m->d_ids + kMaxTopK + 1, sizeof(int), hipMemcpyDeviceToHost, m->stream) != hipSuccess ||
+      hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the sampled id back failed");
+  return check_error_word(m->error);
 }
 
 int shainet_llama_model_write_logits(shainet_llama_model *m, const float *logits) {

@@ -128,6 +128,9 @@ _SIGNATURES = {
                                                       C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "shainet_llama_model_repetition_penalty": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_double]),
     "shainet_llama_model_topk": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), _f32p, C.POINTER(C.c_int)]),
+    "shainet_llama_model_sample": (C.c_int, [C.c_void_p, C.c_int, C.c_double, C.c_double, C.POINTER(C.c_int)]),
+    "shainet_hip_matmul_f32": (C.c_int, [C.c_void_p, C.c_longlong, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                         C.c_int, C.c_void_p]),
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_mfma_f32_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_longlong), C.c_void_p]),
@@ -265,6 +268,24 @@ def describe_plan(num_heads, num_kv_heads, head_dim, start_pos, new_tokens):
     plan = (C.c_int * 8)()
     _check(lib().shainet_attn_describe_plan(num_heads, num_kv_heads, head_dim, n, sp, nt, plan))
     return dict(zip(PLAN_FIELDS, (int(v) for v in plan)))
+
+
+def matmul(x, w, res=None, out=None, stream=None):
+    """y = x @ w (+ res) on torch CUDA float32 tensors: x [T, K] (rows may be strided), w [K, N]."""
+    import torch
+
+    assert x.is_cuda and w.is_cuda and x.dtype == w.dtype == torch.float32 and w.is_contiguous()
+    assert x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[0] and x.stride(1) == 1
+    T, K = x.shape
+    N = w.shape[1]
+    if out is None:
+        out = torch.empty((T, N), device=x.device, dtype=torch.float32)
+    assert out.is_contiguous() and tuple(out.shape) == (T, N)
+    if res is not None:
+        assert res.is_contiguous() and tuple(res.shape) == (T, N)
+    _check(lib().shainet_hip_matmul_f32(x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(res), out.data_ptr(), T, K, N,
+                                        stream))
+    return out
 
 
 def stream_copy(src, dst, workgroups=4096, stream=None):
@@ -771,6 +792,13 @@ class Sampler:
         _check(lib().shainet_llama_model_topk(model._h, k, ids.ctypes.data_as(C.POINTER(C.c_int)),
                                               vals.ctypes.data_as(_f32p), C.byref(n)))
         return ids[:n.value], vals[:n.value]
+
+    def sample_on_device(self, model, r=None):
+        """Sampler#sample with every step on the device; r: the uniform draw (default: one from `rng`)."""
+        tok = C.c_int()
+        r = self.rng.random() if r is None else r
+        _check(lib().shainet_llama_model_sample(model._h, self.top_k, self.temperature, r, C.byref(tok)))
+        return tok.value
 
     def sample(self, model):
         import math

@@ -63,7 +63,7 @@ def _oracle_forward(ob, p, eps, x):
     (64, 8, 4, None, 96, False, False, [6, 1, 1]),        # odd sizes, generic attention kernel (hd 8)
     (128, 8, 2, 64, 344, True, True, [20, 3, 1, 17, 1]),  # explicit head_dim, QK-norm, biases, ff % 8 == 0 only
     (256, 8, 8, 128, 1024, True, False, [33, 1, 1]),
-    (30, 3, 1, None, 50, False, False, [4, 1]),           # widths not multiples of 4: scalar paths, rocBLAS
+    (30, 3, 1, None, 50, False, False, [4, 1]),           # widths not multiples of 4: the plain product kernel
 ])
 def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
     blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e6, seed=d + ff, norm=norm, bias=bias)
@@ -146,8 +146,9 @@ def test_qkv_product_with_prep_inside_equals_separate_prep_bit_for_bit(hip, hd, 
             rm.assert_close(y, unfused[f"arr_{i}"], ATOL, RTOL, f"call {i}")
 
 
-def test_block_many_rows_both_library_gemms(hip):
-    # more than 16 rows: rocBLAS below 256 rows of a small weight matrix, hipBLASLt from 256 rows on
+def test_block_many_rows_take_the_mfma_product(hip):
+    # more than 16 rows: every projection runs the MFMA product kernel (344 = 10.75 steps of 32 along K
+    # for the down projection: the guarded variant; 128 and 256 columns: whole and ragged tiles)
     blk, ob, p, r, eps = _block_pair(hip, 128, 8, 2, 64, 344, 1e4, seed=5, norm=True, bias=True)
     for T in (40, 255, 256, 300):
         x = r.standard_normal((T, 128)).astype(np.float32)
@@ -155,10 +156,63 @@ def test_block_many_rows_both_library_gemms(hip):
     assert blk.cache_len == ob.cache_len == 851
 
 
+@pytest.mark.parametrize("T,K,N,res,stride", [
+    (17, 32, 64, False, None),       # one ragged tile, one step along K
+    (40, 128, 128, True, None),
+    (129, 64, 132, False, None),     # two row tiles, columns past a tile edge
+    (300, 344, 128, True, None),     # K not a multiple of 32: the guarded loads
+    (255, 2048, 3072, False, None),  # the q | k | v product of the 1B shape: K cut into chunks
+    (100, 30, 50, False, None),      # nothing a multiple of 4: the plain kernel
+    (33, 128, 96, False, 160),       # rows of x at a stride
+    (5, 256, 64, True, None),        # few rows: the split GEMV behind the same entry point
+    (24, 8192, 2048, True, None),    # the down projection of the 1B shape, 16 chunks along K
+])
+def test_matmul_matches_oracle(hip, T, K, N, res, stride):
+    """The projection product by itself against SimpleMatrix#* as the oracle restates it (fp64
+    accumulation, one rounding); the device accumulates in fp32, in another order."""
+    import torch
+
+    from shainet_amd import hip as binding
+
+    r = np.random.default_rng(T + K + N)
+    x = r.standard_normal((T, stride or K)).astype(np.float32)
+    w = (r.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    rs = r.standard_normal((T, N)).astype(np.float32) if res else None
+    want = orc.matmul(np.ascontiguousarray(x[:, :K]), w)
+    if res:
+        want = (want.astype(np.float64) + rs).astype(np.float32)  # SimpleMatrix#+ (simple_matrix.cr:39-48)
+    xd = torch.from_numpy(x).cuda()[:, :K]
+    got = binding.matmul(xd, torch.from_numpy(w).cuda(), torch.from_numpy(rs).cuda() if res else None)
+    torch.cuda.synchronize()
+    rm.assert_close(got.cpu().numpy(), want, ATOL, RTOL, f"T={T} K={K} N={N}")
+    # the same call again gives the same bits (partial products are added in a fixed order)
+    again = binding.matmul(xd, torch.from_numpy(w).cuda(), torch.from_numpy(rs).cuda() if res else None)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+
+
+def test_matmul_full_tiles_llama1b_prefill_shapes(hip):
+    # 512 rows of the four products of a Llama-3.2-1B block against torch in fp64 (the oracle's scalar
+    # loop would take minutes here; it is pinned against the same fp64 product in tests/test_oracle_pins.py)
+    import torch
+
+    from shainet_amd import hip as binding
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    for K, N in ((2048, 3072), (2048, 2048), (2048, 16384), (8192, 2048)):
+        x = torch.randn((512, K), generator=g, device="cuda")
+        w = torch.randn((K, N), generator=g, device="cuda") / K ** 0.5
+        got = binding.matmul(x, w)
+        want = (x.double() @ w.double()).float()
+        torch.cuda.synchronize()
+        err = (got - want).abs()
+        assert bool((err <= ATOL + RTOL * want.abs()).all()), f"K={K} N={N}: max err {err.max().item():.2e}"
+
+
 def test_block_llama1b_shape_prefill_and_decode(hip):
     # Llama-3.2-1B block: hidden 2048, 32 Q / 8 KV heads, head_dim 64, ff 8192, theta 5e5
     blk, ob, p, r, eps = _block_pair(hip, 2048, 32, 8, None, 8192, 500000.0, seed=7, wscale=0.02, eps=1e-5)
-    x = r.standard_normal((24, 2048)).astype(np.float32)       # library GEMMs: rocBLAS (QKV, O), hipBLASLt (gate|up, down)
+    x = r.standard_normal((24, 2048)).astype(np.float32)       # MFMA product kernel, K cut into chunks (few tiles)
     rm.assert_close(blk.forward_cached(x), _oracle_forward(ob, p, eps, x), ATOL, RTOL, "prefill 24")
     for i in range(2):                                         # split GEMV projections
         x = r.standard_normal((1, 2048)).astype(np.float32)
@@ -393,6 +447,30 @@ def test_device_repetition_penalty_and_sample_match_oracle(hip, sampler_model):
     for r in (0.0, 0.03, 0.25, 0.5, 0.77, 0.999999):
         s.rng = Fixed(r)
         assert s.sample(m) == orc.sample(want, 40, 0.6, r)
+        assert s.sample_on_device(m) == orc.sample(want, 40, 0.6, r)  # softmax and pick on the device too
+
+
+def test_device_sample_distribution_and_edges(hip, sampler_model):
+    """shainet_llama_model_sample against orc_sample over many draws and temperatures (the device's
+    fp64 exp may differ from libm's in the last bit: a draw within 1e-12 of a step of the cumulative
+    distribution could pick the neighbour, which none of these is), and its edge cases."""
+    m = sampler_model
+    rng = np.random.default_rng(9)
+    row = _row(rng, m.vocab, True)
+    m.set_logits(row)
+    for k, t in ((1, 1.0), (5, 0.3), (40, 1.0), (256, 2.5)):
+        s = hip.Sampler(temperature=t, top_k=k)
+        for r in rng.random(40):
+            assert s.sample_on_device(m, float(r)) == orc.sample(row, k, t, float(r)), (k, t, r)
+    small = hip.LlamaModel(4, 8, 1, 1, 8)
+    small.set_logits([NAN] * 4)
+    assert hip.Sampler(top_k=3).sample_on_device(small, 0.5) == 0          # all-NaN row (sampler.cr:121)
+    small.set_logits([0.0, 5.0, NAN, 5.0])
+    assert hip.Sampler(top_k=2, temperature=1.0).sample_on_device(small, 0.49) == 1   # two equal survivors: lower id first
+    assert hip.Sampler(top_k=2, temperature=1.0).sample_on_device(small, 0.51) == 3
+    assert hip.Sampler(top_k=4, temperature=1.0).sample_on_device(small, 0.9999999) == 0  # only three are eligible
+    with pytest.raises(hip.ArgumentError):
+        hip.Sampler(top_k=300).sample_on_device(small, 0.5)
 
 
 # ---- HFLoader.load_llama on the device --------------------------------------------------------
