@@ -132,6 +132,15 @@ class Workload:
             for s, L in enumerate(self.lens):
                 self.cache.truncate(s, L)
         warm_ms = (time.perf_counter() - t_w) * 1e3
+        # what a call costs the host: a few calls into an empty queue, not waited for
+        n_host = min(16, steps)
+        t0 = time.perf_counter()
+        for i in range(n_host):
+            step(i)
+        host_us = (time.perf_counter() - t0) / n_host * 1e6
+        ctx.sync()
+        for s, L in enumerate(self.lens):
+            self.cache.truncate(s, L)
         t0 = time.perf_counter()
         for i in range(steps):
             step(i)
@@ -155,7 +164,7 @@ class Workload:
         pct = [float(x) * 1e3 for x in np.percentile(samples, (10, 50, 90))] if launches else [0.0] * 3
         return {"workload": self.name, "us_per_step": us, "kernel_us": kus, "kernel_us_p10": pct[0],
                 "kernel_us_p50": pct[1], "kernel_us_p90": pct[2], "launches": launches,
-                "warmup_launches": n_w, "warmup_ms": warm_ms,
+                "warmup_launches": n_w, "warmup_ms": warm_ms, "host_us_per_call": host_us,
                 "bytes_per_step": b_wall, "step_gbps": b_wall / us / 1e3, "kernel_gbps": b_prof / kus / 1e3,
                 "kernel_bytes": b_prof, "frac_of_hbm_peak": b_prof / kus / 1e3 / HBM_PEAK_GBPS}
 

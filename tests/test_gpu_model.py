@@ -255,6 +255,18 @@ def test_block_device_pointers_match_host_pointers(hip):
     got = blk.forward_cached(torch.from_numpy(x).cuda())
     torch.cuda.synchronize()  # the call is asynchronous on the block's stream
     np.testing.assert_array_equal(got.cpu().numpy(), want)
+    # the no-cache call (LlamaBlock#forward, attention_full_gpu: llama_block.cr:533-582) with device
+    # pointers, for few rows (split GEMV) and many (MFMA product): same bits as with host pointers,
+    # and the cache is left alone
+    for T in (5, 40):
+        xf = r.standard_normal((T, 128)).astype(np.float32)
+        want_full = blk.forward(xf)
+        got_full = blk.forward(torch.from_numpy(xf).cuda())
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(got_full.cpu().numpy(), want_full)
+        rm.assert_close(want_full, ob.forward(xf, p["norm1"], p["norm2"], eps, p["gate"], p["up"], p["down"], False),
+                        ATOL, RTOL, f"no-cache forward T={T}")
+    assert blk.cache_len == 5
 
 
 def test_block_argument_errors(hip):
