@@ -97,6 +97,31 @@ struct DevBuf {
   }
 };
 
+// Grow-only pinned host buffer: host-pointer calls stage their rows through it, so that each
+// copy to or from the device is one asynchronous DMA instead of the runtime's staged copy of
+// pageable memory.
+struct PinBuf {
+  float *p = nullptr;
+  size_t cap = 0;  // floats
+  int reserve(size_t n) {
+    if (n <= cap) return SHAINET_HIP_OK;
+    size_t want = cap ? cap : 4096;
+    while (want < n) want *= 2;
+    float *np = nullptr;
+    hipError_t e = hipHostMalloc((void **)&np, want * sizeof(float), hipHostMallocDefault);
+    if (e != hipSuccess) return hip_fail(e, "hipHostMalloc");
+    if (p) (void)hipHostFree(p);
+    p = np;
+    cap = want;
+    return SHAINET_HIP_OK;
+  }
+  void release() {
+    if (p) (void)hipHostFree(p);
+    p = nullptr;
+    cap = 0;
+  }
+};
+
 }  // namespace
 
 struct shainet_attn_ctx {
@@ -111,6 +136,7 @@ struct shainet_attn_ctx {
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
+  PinBuf pin_in, pin_out;  // host-pointer calls: q | k | v rows on their way in, the result on its way out
   // decode split: a word per partial slot that says when it is complete (zero between launches)
   unsigned *part_flag = nullptr;
   size_t part_flag_cap = 0;
@@ -454,6 +480,8 @@ int shainet_attn_destroy(shainet_attn_ctx *c) {
   if (c->part_flag) (void)hipFree(c->part_flag);
   for (hipEvent_t ev : c->prof_events) (void)hipEventDestroy(ev);
   for (DevBuf *b : {&c->q_rot, &c->partials, &c->in_q, &c->in_k, &c->in_v, &c->out}) b->release();
+  c->pin_in.release();
+  c->pin_out.release();
   free_error_word(c->own_error);
   delete c;
   return SHAINET_HIP_OK;
@@ -697,11 +725,17 @@ int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, 
   float *dout = out;
   if (mem == SHAINET_HIP_MEM_HOST) {
     if ((rc = c->in_q.reserve(q_floats)) || (rc = c->in_k.reserve(kv_floats)) ||
-        (rc = c->in_v.reserve(kv_floats)) || (rc = c->out.reserve(q_floats)))
+        (rc = c->in_v.reserve(kv_floats)) || (rc = c->out.reserve(q_floats)) ||
+        (rc = c->pin_in.reserve(q_floats + 2 * kv_floats)) || (rc = c->pin_out.reserve(q_floats)))
       return rc;
-    HIP_TRY(hipMemcpyAsync(c->in_q.p, q, q_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
-    HIP_TRY(hipMemcpyAsync(c->in_k.p, k, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
-    HIP_TRY(hipMemcpyAsync(c->in_v.p, v, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    // (the last call's copies are done: every host-pointer call ends with a wait)
+    float *pq = c->pin_in.p, *pk = pq + q_floats, *pv = pk + kv_floats;
+    memcpy(pq, q, q_floats * sizeof(float));
+    memcpy(pk, k, kv_floats * sizeof(float));
+    memcpy(pv, v, kv_floats * sizeof(float));
+    HIP_TRY(hipMemcpyAsync(c->in_q.p, pq, q_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(hipMemcpyAsync(c->in_k.p, pk, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(hipMemcpyAsync(c->in_v.p, pv, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
     dq = c->in_q.p;
     dk = c->in_k.p;
     dv = c->in_v.p;
@@ -734,8 +768,9 @@ int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, 
   for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
   c->last_rows = ws ? 0 : rows;  // shainet_attn_last_q_rot reads the context's own buffer
   if (mem == SHAINET_HIP_MEM_HOST) {
-    HIP_TRY(hipMemcpyAsync(out, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipMemcpyAsync(c->pin_out.p, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
+    memcpy(out, c->pin_out.p, q_floats * sizeof(float));
     return check_error_word(c->error);
   }
   return SHAINET_HIP_OK;

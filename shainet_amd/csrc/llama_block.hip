@@ -44,6 +44,7 @@ struct shainet_llama_attn {
   int *shared_error = nullptr;  // the error word of the model that owns this block, if one does
   Projector proj;
   DevF x, qkv, attn, out;
+  PinnedF x_pin, out_pin;  // host-pointer calls stage their rows here
 };
 
 namespace {
@@ -191,6 +192,8 @@ int shainet_llama_attn_destroy(shainet_llama_attn *l) {
   for (float *p : {l->w_qkv, l->w_o})
     if (p) (void)hipFree(p);
   for (DevF *b : {&l->x, &l->qkv, &l->attn, &l->out}) b->release();
+  l->x_pin.release();
+  l->out_pin.release();
   delete l;
   return SHAINET_HIP_OK;
 }
@@ -257,14 +260,17 @@ static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_toke
   int rc = ensure_context(l);  // raises what add_bias! / apply_head_rmsnorm! raise (llama_block.cr:587, 618)
   if (rc) return rc;
   const size_t xd = (size_t)new_tokens * l->d_model;
-  if (!l->x.reserve(xd) || !l->out.reserve(xd)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (!l->x.reserve(xd) || !l->out.reserve(xd) || !l->x_pin.reserve(xd) || !l->out_pin.reserve(xd))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   hipStream_t stream = (hipStream_t)shainet_attn_stream(l->ctx);
-  if (hipMemcpyAsync(l->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
+  memcpy(l->x_pin.p, x, xd * sizeof(float));  // the last call's copies are done: every host-pointer call ends with a wait
+  if (hipMemcpyAsync(l->x.p, l->x_pin.p, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
   if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p, Fused(), nullptr, no_cache))) return rc;
-  if (hipMemcpyAsync(out, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+  if (hipMemcpyAsync(l->out_pin.p, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
+  memcpy(out, l->out_pin.p, xd * sizeof(float));
   return check_error_word(shainet_attn_error_word(l->ctx));
 }
 
@@ -280,6 +286,7 @@ struct shainet_llama_block {
   float *norm1 = nullptr, *norm2 = nullptr;         // device gamma [d_model]; null = ones (rms_norm.cr:10)
   float *gate_up = nullptr, *down = nullptr;        // device [d_model, 2*ff] (gate | up) and [ff, d_model]
   DevF x, h, hidden, out;
+  PinnedF x_pin, out_pin;  // host-pointer calls stage their rows here
 };
 
 namespace {
@@ -395,6 +402,8 @@ int shainet_llama_block_destroy(shainet_llama_block *b) {
   for (float *p : {b->norm1, b->norm2, b->gate_up, b->down})
     if (p) (void)hipFree(p);
   for (DevF *f : {&b->x, &b->h, &b->hidden, &b->out}) f->release();
+  b->x_pin.release();
+  b->out_pin.release();
   delete b;
   return SHAINET_HIP_OK;
 }
@@ -453,14 +462,17 @@ static int block_forward_any(shainet_llama_block *b, const float *x, int new_tok
   int rc = ensure_context(b->attn);
   if (rc) return rc;
   const size_t xd = (size_t)new_tokens * b->d_model;
-  if (!b->x.reserve(xd) || !b->out.reserve(xd)) return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (!b->x.reserve(xd) || !b->out.reserve(xd) || !b->x_pin.reserve(xd) || !b->out_pin.reserve(xd))
+    return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   hipStream_t stream = (hipStream_t)shainet_attn_stream(b->attn->ctx);
-  if (hipMemcpyAsync(b->x.p, x, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
+  memcpy(b->x_pin.p, x, xd * sizeof(float));
+  if (hipMemcpyAsync(b->x.p, b->x_pin.p, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
   if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p, no_cache))) return rc;
-  if (hipMemcpyAsync(out, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+  if (hipMemcpyAsync(b->out_pin.p, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
+  memcpy(out, b->out_pin.p, xd * sizeof(float));
   return check_error_word(shainet_attn_error_word(b->attn->ctx));
 }
 

@@ -48,6 +48,16 @@ struct DevF {
   void release();
 };
 
+// Grow-only pinned host buffer: host-pointer calls stage their rows through it, so that the
+// copies to and from the device run as one asynchronous DMA each instead of the runtime's
+// staged copy of pageable memory.
+struct PinnedF {
+  float *p = nullptr;
+  size_t cap = 0;
+  bool reserve(size_t n);
+  void release();
+};
+
 // What rides along with a projection y = x W.
 struct Fused {
   int epilogue = 0;            // kGemvPlain, kGemvResidual (y = res + x W) or kGemvSwiglu (W = gate | up, [K, 2N])

@@ -35,6 +35,27 @@ bool DevF::reserve(size_t n) {
   return true;
 }
 
+bool PinnedF::reserve(size_t n) {
+  if (n <= cap) return true;
+  size_t want = cap ? cap : 4096;
+  while (want < n) want *= 2;
+  float *np = nullptr;
+  if (hipHostMalloc((void **)&np, want * sizeof(float), hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  if (p) (void)hipHostFree(p);
+  p = np;
+  cap = want;
+  return true;
+}
+
+void PinnedF::release() {
+  if (p) (void)hipHostFree(p);
+  p = nullptr;
+  cap = 0;
+}
+
 void DevF::release() {
   if (p) (void)hipFree(p);
   p = nullptr;
