@@ -244,6 +244,23 @@ module SHAInet
       check fn.call(ctx, cache, Pointer(Int32).null, pointerof(nt), 1, q, k, v, out_ptr)
     end
 
+    # Decode steps with the cached lengths on the device (launches that never change: a step can be
+    # recorded into a HIP graph and replayed): shainet_kv_cache_lengths_to_device before the first
+    # step, shainet_attn_decode_step per token, shainet_kv_cache_lengths_from_device after the last.
+    def kv_cache_lengths_to_device(cache : Handle)
+      check Proc(Handle, Int32).new(sym("shainet_kv_cache_lengths_to_device"), Pointer(Void).null).call(cache)
+    end
+
+    def kv_cache_lengths_from_device(cache : Handle)
+      check Proc(Handle, Int32).new(sym("shainet_kv_cache_lengths_from_device"), Pointer(Void).null).call(cache)
+    end
+
+    def attn_decode_step(ctx : Handle, cache : Handle, n_seqs : Int32,
+                         q : Pointer(Float32), k : Pointer(Float32), v : Pointer(Float32), out_ptr : Pointer(Float32))
+      fn = Proc(Handle, Handle, Int32, Pointer(Float32), Pointer(Float32), Pointer(Float32), Pointer(Float32), Int32).new(sym("shainet_attn_decode_step"), Pointer(Void).null)
+      check fn.call(ctx, cache, n_seqs, q, k, v, out_ptr)
+    end
+
     def attn_sync(ctx : Handle)
       check Proc(Handle, Int32).new(sym("shainet_attn_sync"), Pointer(Void).null).call(ctx)
     end

@@ -52,7 +52,8 @@ module SHAInet
 
     {% for name in %w(sym malloc memcpy kv_cache_append_f32 attention_kv_f32 attn_create attn_set_bias
                      kv_cache_create kv_cache_clear kv_cache_len kv_cache_capacity kv_cache_reserve
-                     attn_forward attn_forward_noalloc attn_sync rope_apply matmul_f32 check) %}
+                     attn_forward attn_forward_noalloc attn_decode_step kv_cache_lengths_to_device
+                     kv_cache_lengths_from_device attn_sync rope_apply matmul_f32 check) %}
       def {{name.id}}(*args)
         raise "HIP disabled"
       end

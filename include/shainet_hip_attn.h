@@ -169,6 +169,35 @@ int shainet_attn_forward_noalloc(shainet_attn_ctx *ctx, shainet_kv_cache *cache,
                                  const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                                  float *out);
 
+/* Decode steps whose launches never change, for callers that record a step once and replay it (a HIP
+ * graph): one new row for each of the first n_seqs sequences of a cache, the same arithmetic as
+ * shainet_attn_forward with new_tokens all 1 (LlamaBlock#attention_cached_cpu with one row,
+ * llama_block.cr:246-299).  Nothing the three kernels of a step are launched with depends on how
+ * many rows the cache holds: the lengths live in device memory, a one-wavefront kernel at the head
+ * of each step reads them, lays out the split of the keys for the other two kernels and adds one
+ * to each length.  The step allocates nothing and copies nothing; it has no counterpart in the
+ * reference, whose cache length is a host integer (llama_block.cr:288-289).
+ *
+ * shainet_kv_cache_lengths_to_device: allocates what the steps need (first call), extends the
+ *   context's cos/sin table to the cache's capacity and copies the host's lengths to the device.
+ *   Call it after anything that changes the lengths on the host (shainet_attn_forward, fill,
+ *   clear, truncate) or the capacity (reserve), before the next step; not while capturing.
+ * shainet_attn_decode_step: q [n_seqs, num_heads*head_dim], k, v [n_seqs, num_kv_heads*head_dim],
+ *   out like q; device pointers, asynchronous on the context's stream.  head_dim 64 or 128.
+ *   A step that finds a sequence at the cache's capacity appends nothing, writes no output and
+ *   leaves the lengths alone, and so do the steps after it; shainet_kv_cache_lengths_from_device
+ *   (or shainet_attn_sync) then returns SHAINET_HIP_ERR_CAPACITY.
+ * shainet_kv_cache_lengths_from_device: waits for the stream and copies the device's lengths
+ *   back, so that shainet_kv_cache_len and the other entry points see the rows the steps appended.
+ * Between the two copies the host's lengths are stale: use no other entry point on the cache.
+ * A recorded step holds the addresses of the cache, of the context's cos/sin table, bias and
+ * QK-norm weights: record it again after shainet_kv_cache_reserve, shainet_attn_set_bias, or a
+ * call on another cache of the same context that reaches beyond the table's positions. */
+int shainet_kv_cache_lengths_to_device(shainet_kv_cache *cache);
+int shainet_kv_cache_lengths_from_device(shainet_kv_cache *cache);
+int shainet_attn_decode_step(shainet_attn_ctx *ctx, shainet_kv_cache *cache, int n_seqs, const float *q,
+                             const float *k, const float *v, float *out);
+
 /* Copy of the rotated query rows of the last shainet_attn_forward call
  * ([sum new_tokens, num_heads*head_dim], host): lets a test check RoPE positions
  * and QK-norm of Q exactly (llama_block.cr:332-344). */

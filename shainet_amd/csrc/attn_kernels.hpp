@@ -48,9 +48,12 @@ struct PrepArgs {
   float *kc, *vc;
 };
 
+struct DecodeDevicePlan;
 // bias -> QK-norm -> RoPE -> append (K rotated, V as is); rotated Q to q_rot.
+// dev != nullptr: one new row for each of st.n_seqs sequences, their positions read from
+// *dev (device memory) instead of st.
 hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, int total_tokens,
-                       hipStream_t stream);
+                       hipStream_t stream, const DecodeDevicePlan *dev = nullptr);
 
 // Which attention kernel a call uses.
 enum class Path { kDecodeSplitK, kPrefillMfma, kGeneric };
@@ -81,6 +84,26 @@ struct DecodePlan {
 };
 // wg_target: 0 = default
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target);
+
+// The same plan made on the device, for decode steps whose launches must not change from step to
+// step (a captured graph that is replayed): a step of one new row for each of the first n_seqs
+// slots of a cache.  decode_plan_kernel reads the cached lengths from device memory, writes
+// this record (also device memory) for the prep and decode kernels of the step, and adds the
+// step's rows to the lengths.  The launches then depend on nothing but the number of
+// sequences and the head geometry: a fixed 256 workgroups, kDevicePlanSlots(...) partial slots.
+struct DecodeDevicePlan {
+  SeqTable st;
+  int tiles_per_wg;
+  SpanTable spans;
+  int total_tiles;
+  int skip;  // a sequence would outgrow the cache or the cos/sin table: the step's kernels do nothing
+};
+constexpr int kDevicePlanWorkgroups = 256;
+inline int device_plan_slots(int n_seqs, int KV) { return kDevicePlanWorkgroups + n_seqs * KV; }
+// lens: cached length per slot (device); rope_positions: positions the cos/sin table covers;
+// error: set to 2 when the step is skipped.
+hipError_t launch_decode_plan(int *lens, int n_seqs, const Shape &sh, int rope_positions, DecodeDevicePlan *out,
+                              int *error, hipStream_t stream);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
 size_t decode_flag_words(const DecodePlan &p);
 
@@ -102,8 +125,11 @@ struct DecodeArgs {
   unsigned *flag_set;
   int spin_limit;
 };
+// dev != nullptr: st gives the number of sequences only, p the grid (kDevicePlanWorkgroups), the
+// slots and the columns; everything that depends on the cached lengths is read from *dev.
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
-                         hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr);
+                         hipStream_t stream, hipEvent_t before = nullptr, hipEvent_t after = nullptr,
+                         const DecodeDevicePlan *dev = nullptr);
 // Key splits of a prefill launch: 1 when the row blocks alone fill the chip, more
 // when they do not (few new rows on a long cached prefix); each split leaves
 // partial rows in `partials` (prefill_partial_floats) and a second kernel merges.

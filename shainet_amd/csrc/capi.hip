@@ -51,7 +51,12 @@ void free_error_word(int *w) {
 
 int check_error_word(int *w) {
   if (!w || *(volatile int *)w == 0) return SHAINET_HIP_OK;
+  const int what = *(volatile int *)w;
   *(volatile int *)w = 0;
+  if (what == 2)
+    return fail(SHAINET_HIP_ERR_CAPACITY,
+                "a decode step found a sequence at the capacity of its cache or at the end of the context's "
+                "cos/sin table: that step and the steps after it appended nothing and wrote no output");
   return fail(SHAINET_HIP_ERR_RUNTIME, "a kernel gave up waiting for the partial results of other workgroups; the results of the calls on this handle since its last wait are invalid and it must be destroyed");
 }
 
@@ -153,11 +158,24 @@ struct shainet_attn_ctx {
   std::vector<hipEvent_t> prof_events;  // start, stop, start, stop, ...
 };
 
+// What shainet_attn_decode_step works with: all of it allocated by shainet_kv_cache_lengths_to_device,
+// none of it by the step.
+struct StepState {
+  int *d_len = nullptr;               // [batch] cached rows per slot, as the device counts them
+  int *pin_len = nullptr;             // [batch] pinned staging for both directions
+  DecodeDevicePlan *d_plan = nullptr; // rewritten by every step
+  float *q_rot = nullptr;             // [batch, H, hd]
+  float *partials = nullptr;          // device_plan_slots(batch, KV) slots of g columns
+  unsigned *flags = nullptr;          // zero between launches
+  int cap = 0;                        // the capacity the buffers above were laid out for
+};
+
 struct shainet_kv_cache {
   shainet_attn_ctx *ctx;
   int batch, cap;
   float *k = nullptr, *v = nullptr;
   std::vector<int> len;
+  StepState step;
 };
 
 namespace {
@@ -540,6 +558,12 @@ int shainet_kv_cache_create(shainet_kv_cache **out, shainet_attn_ctx *ctx, int b
 int shainet_kv_cache_destroy(shainet_kv_cache *kc) {
   if (!kc) return SHAINET_HIP_OK;
   if (kc->ctx) (void)hipStreamSynchronize(kc->ctx->stream);
+  if (kc->step.d_len) (void)hipFree(kc->step.d_len);
+  if (kc->step.pin_len) (void)hipHostFree(kc->step.pin_len);
+  if (kc->step.d_plan) (void)hipFree(kc->step.d_plan);
+  if (kc->step.q_rot) (void)hipFree(kc->step.q_rot);
+  if (kc->step.partials) (void)hipFree(kc->step.partials);
+  if (kc->step.flags) (void)hipFree(kc->step.flags);
   if (kc->k) (void)hipFree(kc->k);
   if (kc->v) (void)hipFree(kc->v);
   delete kc;
@@ -839,6 +863,119 @@ extern "C" int shainet_attn_forward_noalloc(shainet_attn_ctx *c, shainet_kv_cach
   HIP_TRY(hipGetLastError());
   return forward_core(c, kc, seq_ids, new_tokens, n_seqs, q, k, v, (long long)c->H * c->hd, (long long)c->KV * c->hd,
                       (long long)c->KV * c->hd, out, SHAINET_HIP_MEM_DEVICE, &ws);
+}
+
+// ---- decode steps whose launches never change ------------------------------------------------
+
+namespace {
+DecodePlan step_launch_plan(const shainet_attn_ctx *c, int n_seqs) {
+  DecodePlan p;
+  memset(&p, 0, sizeof p);
+  p.n_wgs = kDevicePlanWorkgroups;
+  p.n_slots = device_plan_slots(n_seqs, c->KV);
+  p.cols = c->g;
+  return p;
+}
+}  // namespace
+
+extern "C" int shainet_kv_cache_lengths_to_device(shainet_kv_cache *kc) {
+  if (!kc) return fail(SHAINET_HIP_ERR_ARGUMENT, "cache is null");
+  shainet_attn_ctx *c = kc->ctx;
+  if ((c->hd != 64 && c->hd != 128) || c->g > 16)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps need head_dim 64 or 128 and at most 16 query heads per kv head");
+  if (kc->batch > SHAINET_HIP_MAX_BATCH)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps take caches of at most %d sequences", SHAINET_HIP_MAX_BATCH);
+  StepState &st = kc->step;
+  if (!st.d_len) {
+    const DecodePlan p = step_launch_plan(c, kc->batch);
+    const size_t flag_words = decode_flag_words(p);
+    HIP_TRY(hipMalloc((void **)&st.d_len, kc->batch * sizeof(int)));
+    HIP_TRY(hipHostMalloc((void **)&st.pin_len, kc->batch * sizeof(int), hipHostMallocDefault));
+    HIP_TRY(hipMalloc((void **)&st.d_plan, sizeof(DecodeDevicePlan)));
+    HIP_TRY(hipMalloc((void **)&st.q_rot, (size_t)kc->batch * c->H * c->hd * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&st.partials, decode_partial_floats(shape_of(c, kc->cap), p) * sizeof(float)));
+    HIP_TRY(hipMalloc((void **)&st.flags, flag_words * sizeof(unsigned)));
+    HIP_TRY(hipMemsetAsync(st.d_plan, 0, sizeof(DecodeDevicePlan), c->stream));
+    HIP_TRY(hipMemsetAsync(st.flags, 0, flag_words * sizeof(unsigned), c->stream));
+    if (!c->error) {
+      c->error = c->own_error = alloc_error_word();
+      if (!c->error) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+    }
+  }
+  // the cos/sin table must reach as far as the cache: a step cannot grow it
+  if (int rc = ensure_rope_table(c, kc->cap)) return rc;
+  for (int s = 0; s < kc->batch; ++s) st.pin_len[s] = kc->len[s];
+  HIP_TRY(hipMemcpyAsync(st.d_len, st.pin_len, kc->batch * sizeof(int), hipMemcpyHostToDevice, c->stream));
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  st.cap = kc->cap;
+  return SHAINET_HIP_OK;
+}
+
+extern "C" int shainet_kv_cache_lengths_from_device(shainet_kv_cache *kc) {
+  if (!kc) return fail(SHAINET_HIP_ERR_ARGUMENT, "cache is null");
+  StepState &st = kc->step;
+  if (!st.d_len) return fail(SHAINET_HIP_ERR_ARGUMENT, "shainet_kv_cache_lengths_to_device has not been called");
+  shainet_attn_ctx *c = kc->ctx;
+  HIP_TRY(hipMemcpyAsync(st.pin_len, st.d_len, kc->batch * sizeof(int), hipMemcpyDeviceToHost, c->stream));
+  HIP_TRY(hipStreamSynchronize(c->stream));
+  for (int s = 0; s < kc->batch; ++s) {
+    if (st.pin_len[s] < 0 || st.pin_len[s] > kc->cap)
+      return fail(SHAINET_HIP_ERR_RUNTIME, "the device holds length %d for sequence %d of a cache of capacity %d",
+                  st.pin_len[s], s, kc->cap);
+    kc->len[s] = st.pin_len[s];
+  }
+  return check_error_word(c->error);
+}
+
+extern "C" int shainet_attn_decode_step(shainet_attn_ctx *c, shainet_kv_cache *kc, int n_seqs, const float *q,
+                                        const float *k, const float *v, float *out) {
+  if (!c || !kc || kc->ctx != c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (!q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  if (n_seqs < 1 || n_seqs > kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", kc->batch);
+  StepState &ss = kc->step;
+  if (!ss.d_len) return fail(SHAINET_HIP_ERR_ARGUMENT, "shainet_kv_cache_lengths_to_device has not been called");
+  if (ss.cap != kc->cap)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "the cache has grown since shainet_kv_cache_lengths_to_device: call it again");
+  const Shape sh = shape_of(c, kc->cap);
+  hipError_t e = launch_decode_plan(ss.d_len, n_seqs, sh, c->rope_positions, ss.d_plan, c->error, c->stream);
+  if (e != hipSuccess) return hip_fail(e, "plan launch");
+  SeqTable st;
+  memset(&st, 0, sizeof st);
+  st.n_seqs = n_seqs;
+  PrepArgs pa;
+  pa.q = q;
+  pa.k = k;
+  pa.v = v;
+  pa.q_stride = (long long)c->H * c->hd;
+  pa.k_stride = pa.v_stride = (long long)c->KV * c->hd;
+  pa.b_q = c->d_bq;
+  pa.b_k = c->d_bk;
+  pa.b_v = c->d_bv;
+  pa.q_norm = c->d_q_norm;
+  pa.k_norm = c->d_k_norm;
+  pa.eps = c->eps;
+  pa.rope_tab = c->d_rope;
+  pa.q_rot = ss.q_rot;
+  pa.kc = kc->k;
+  pa.vc = kc->v;
+  e = launch_prep(pa, st, sh, n_seqs, c->stream, ss.d_plan);
+  if (e != hipSuccess) return hip_fail(e, "prep launch");
+  DecodeArgs d;
+  d.q_rot = ss.q_rot;
+  d.kc = kc->k;
+  d.vc = kc->v;
+  d.out = out;
+  d.partials = ss.partials;
+  d.part_flag = ss.flags;
+  d.flag_set = nullptr;
+  d.error = c->error;
+  d.spin_limit = 0;
+  // (the buffers are sized for the whole cache; a step of fewer sequences uses the front of them)
+  DecodePlan p = step_launch_plan(c, n_seqs);
+  e = launch_decode(d, st, sh, p, c->scale, c->stream, nullptr, nullptr, ss.d_plan);
+  if (e != hipSuccess) return hip_fail(e, "attention launch");
+  c->last_rows = 0;
+  return SHAINET_HIP_OK;
 }
 
 // The owner of a context (a block, a model) makes the context's kernels report into the owner's

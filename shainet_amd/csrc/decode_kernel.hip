@@ -166,13 +166,19 @@ constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each: s
 // (so a launch may be replayed as it is).  error: set when the wait for other workgroups'
 // partials was given up, after spin_limit polls.  flag_set: where the marks are written; the
 // same as part_flag except in the test of that give-up, which sends them elsewhere.
-template <int HD, int NW>
+// DEV: the sequence table and the spans come from *dev (device memory, written by
+// decode_plan_kernel earlier on the stream) instead of from the kernel arguments.
+template <int HD, int NW, bool DEV>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
-    int spin_limit, int *error, SeqTable st, Shape sh, int tiles_per_wg, SpanTable sp, int total_tiles, int n_slots, int pstride,
-    float c, unsigned rotate) {
+    int spin_limit, int *error, SeqTable st_arg, Shape sh, int tiles_per_wg_arg, SpanTable sp_arg, int total_tiles_arg,
+    int n_slots, int pstride, float c, unsigned rotate, const DecodeDevicePlan *__restrict__ dev) {
   using C = DecodeCfg<HD>;
+  const SeqTable &st = DEV ? dev->st : st_arg;
+  const SpanTable &sp = DEV ? dev->spans : sp_arg;
+  const int tiles_per_wg = DEV ? dev->tiles_per_wg : tiles_per_wg_arg;
+  const int total_tiles = DEV ? dev->total_tiles : total_tiles_arg;
   constexpr int NT = C::NT;
   // per wavefront two K tile buffers; after a segment's last tile the wavefront parks its O
   // rows [g][HD] in one while the other already receives the next segment's first tile
@@ -501,6 +507,96 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kDecodeWaves = 4;  // wavefronts per workgroup (eight measured no better)
 
+// Share of each of eight consecutive spans, in thousandths of an equal share, by the XCD the
+// workgroup lands on (index mod 8).  With equal spans the workgroups on odd XCDs finished
+// streaming about 5 % after those on even XCDs on every box traced (3 and 5 last, 0 and 6
+// first; the finer pattern differs from box to box).  SHAINET_HIP_DECODE_SHARES: eight
+// numbers, or "0" for equal spans.  Not worth it for short spans.
+struct Shares {
+  int v[8] = {1050, 950, 1050, 950, 1050, 950, 1050, 950};
+  Shares() {
+    const char *env = getenv("SHAINET_HIP_DECODE_SHARES");
+    if (!env) return;
+    int w[8], n = 0;
+    for (const char *c = env; *c && n < 8;) {
+      char *end;
+      const long x = strtol(c, &end, 10);
+      if (end == c) break;
+      w[n++] = (int)x;
+      c = *end ? end + 1 : end;
+    }
+    for (int i = 0; i < 8; ++i) v[i] = n == 8 && w[i] >= 500 && w[i] <= 1500 ? w[i] : 1000;
+  }
+};
+const Shares &span_shares() {
+  static const Shares shares;
+  return shares;
+}
+
+// Where the spans of eight consecutive workgroups begin within their 8 q tiles, from their shares.
+__host__ __device__ inline void spans_from_shares(const int (&share)[8], int q, SpanTable &spans) {
+  long long sum = 0, acc = 0;
+  for (int i = 0; i < 8; ++i) sum += share[i];
+  for (int i = 0; i <= 8; ++i) {
+    spans.off[i] = q >= 32 ? (int)(acc * 8 * q / sum) : i * q;
+    if (i < 8) acc += share[i];
+  }
+}
+
+struct ShareArg {
+  int v[8];
+};
+
+// plan_decode on the device for one new row per sequence: one wavefront, lane s looks after
+// sequence s.  Reads the cached lengths, writes the record the step's prep and decode kernels
+// read, and adds the step's rows to the lengths.
+__global__ __launch_bounds__(64) void decode_plan_kernel(int *__restrict__ lens, int n_seqs, Shape sh, int rope_positions,
+                                                         ShareArg shares, DecodeDevicePlan *__restrict__ out,
+                                                         int *error) {
+  const int s = threadIdx.x;
+  const bool mine = s < n_seqs;
+  const int start = mine ? lens[s] : 0;
+  const bool fits = !mine || (start >= 0 && start + 1 <= sh.cap && start + 1 <= rope_positions);
+  if (!__all(fits)) {  // nothing is appended: the lengths stay as they are
+    if (s == 0) {
+      out->st.n_seqs = n_seqs;
+      out->tiles_per_wg = 0;
+      out->total_tiles = 0;
+      out->skip = 1;
+      spans_from_shares(shares.v, 0, out->spans);  // all zero: no workgroup finds tiles
+      *error = 2;
+    }
+    return;
+  }
+  const int tiles = mine ? sh.KV * ((start + 1 + 15) >> 4) : 0;
+  int incl = tiles;  // inclusive prefix sum over the lanes
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o);
+    if (s >= o) incl += up;
+  }
+  const int total = __shfl(incl, 63);
+  if (mine) {
+    out->st.slot[s] = s;
+    out->st.start_pos[s] = start;
+    out->st.n_new[s] = 1;
+    out->st.tok_off[s] = s;
+    out->st.work_off[s] = incl - tiles;
+    lens[s] = start + 1;
+  }
+  if (s == 0) {
+    out->st.n_seqs = n_seqs;
+    out->st.tok_off[n_seqs] = n_seqs;
+    out->st.work_off[n_seqs] = total;
+    int q = (total + kDevicePlanWorkgroups - 1) / kDevicePlanWorkgroups;
+    if (q < kDecodeWaves) q = kDecodeWaves;
+    out->tiles_per_wg = q;
+    out->total_tiles = total;
+    out->skip = 0;
+    spans_from_shares(shares.v, q, out->spans);
+  }
+}
+
 }  // namespace
 
 DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
@@ -518,33 +614,7 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
   int q = (p.total_tiles + wg_target - 1) / wg_target;
   if (q < kDecodeWaves) q = kDecodeWaves;
   p.tiles_per_wg = q;
-  // Share of each of eight consecutive spans, in thousandths of an equal share, by the XCD the
-  // workgroup lands on (index mod 8).  With equal spans the workgroups on odd XCDs finished
-  // streaming about 5 % after those on even XCDs on every box traced (3 and 5 last, 0 and 6
-  // first; the finer pattern differs from box to box).  SHAINET_HIP_DECODE_SHARES: eight
-  // numbers, or "0" for equal spans.  Not worth it for short spans.
-  static const struct Shares {
-    int v[8] = {1050, 950, 1050, 950, 1050, 950, 1050, 950};
-    Shares() {
-      const char *env = getenv("SHAINET_HIP_DECODE_SHARES");
-      if (!env) return;
-      int w[8], n = 0;
-      for (const char *c = env; *c && n < 8;) {
-        char *end;
-        const long x = strtol(c, &end, 10);
-        if (end == c) break;
-        w[n++] = (int)x;
-        c = *end ? end + 1 : end;
-      }
-      for (int i = 0; i < 8; ++i) v[i] = n == 8 && w[i] >= 500 && w[i] <= 1500 ? w[i] : 1000;
-    }
-  } shares;
-  long long sum = 0, acc = 0;
-  for (int i = 0; i < 8; ++i) sum += shares.v[i];
-  for (int i = 0; i <= 8; ++i) {
-    p.spans.off[i] = q >= 32 ? (int)(acc * 8 * q / sum) : i * q;
-    if (i < 8) acc += shares.v[i];
-  }
+  spans_from_shares(span_shares().v, q, p.spans);
   // the first workgroup count whose spans cover the stream
   p.n_wgs = (p.total_tiles + q - 1) / q;
   auto begin_of = [&](int w) { return (w >> 3) * 8 * q + p.spans.off[w & 7]; };
@@ -562,15 +632,31 @@ size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
   return (size_t)p.n_slots * p.cols * (sh.hd + 2);
 }
 
+hipError_t launch_decode_plan(int *lens, int n_seqs, const Shape &sh, int rope_positions, DecodeDevicePlan *out,
+                              int *error, hipStream_t stream) {
+  if (!lens || !out || !error || n_seqs < 1 || n_seqs > kMaxSeqs) return hipErrorInvalidValue;
+  ShareArg shares;
+  for (int i = 0; i < 8; ++i) shares.v[i] = span_shares().v[i];
+  hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(64), 0, stream, lens, n_seqs, sh, rope_positions, shares, out,
+                     error);
+  return hipGetLastError();
+}
+
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
-                         hipStream_t stream, hipEvent_t before, hipEvent_t after) {
+                         hipStream_t stream, hipEvent_t before, hipEvent_t after, const DecodeDevicePlan *dev) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
-      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || p.tiles_per_wg < 1 || !d.partials || !d.part_flag || !d.error)
+      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || !d.partials || !d.part_flag || !d.error)
     return hipErrorInvalidValue;
-  for (int s = 0; s < st.n_seqs; ++s)
-    if (st.n_new[s] < 1 || st.n_new[s] * sh.g > 16 || st.n_new[s] * sh.g > p.cols || st.start_pos[s] < 0 ||
-        st.start_pos[s] + st.n_new[s] > sh.cap || st.slot[s] < 0)
+  if (dev) {
+    if (p.n_wgs != kDevicePlanWorkgroups || p.n_slots != device_plan_slots(st.n_seqs, sh.KV) || p.cols < sh.g)
       return hipErrorInvalidValue;
+  } else {
+    if (p.tiles_per_wg < 1) return hipErrorInvalidValue;
+    for (int s = 0; s < st.n_seqs; ++s)
+      if (st.n_new[s] < 1 || st.n_new[s] * sh.g > 16 || st.n_new[s] * sh.g > p.cols || st.start_pos[s] < 0 ||
+          st.start_pos[s] + st.n_new[s] > sh.cap || st.slot[s] < 0)
+        return hipErrorInvalidValue;
+  }
   if (!d.q_rot) return hipErrorInvalidValue;
   unsigned *flag_set = d.flag_set ? d.flag_set : d.part_flag;
   const int spin_limit = d.spin_limit > 0 ? d.spin_limit : kFlagSpinLimit;
@@ -580,21 +666,29 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   // before / after (nullable) receive the kernel's own first and last clock reading, not the
   // time at which the stream reached them: what is between two kernels stays out
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
-  // SHAINET_HIP_DECODE_NO_ROTATE: every workgroup walks its segments from their first tile (for comparison)
-  static const unsigned rotate = getenv("SHAINET_HIP_DECODE_NO_ROTATE") ? 0u : getenv("SHAINET_HIP_DECODE_ROTATE") ? (unsigned)atoi(getenv("SHAINET_HIP_DECODE_ROTATE")) : 0x7fffffffu;
-  const size_t pad = 0;
-  if (sh.hd == 64)
-    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<64, kDecodeWaves>), grid, block, pad, stream, before, after, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
-                          p.total_tiles,
-                          p.n_slots, p.cols, c, rotate);
-  else
-    SHAINET_LAUNCH_TIMED((decode_splitk_kernel<128, kDecodeWaves>), grid, block, pad, stream, before, after, d.q_rot,
-                          d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg, p.spans,
-                          p.total_tiles,
-                          p.n_slots, p.cols, c, rotate);
-  hipError_t e = hipGetLastError();
-  return e;
+  // SHAINET_HIP_DECODE_NO_ROTATE: every workgroup walks its segments from their first tile (for
+  // comparison); SHAINET_HIP_DECODE_ROTATE=n: starts spread over the first n tiles only
+  static const unsigned rotate = getenv("SHAINET_HIP_DECODE_NO_ROTATE") ? 0u
+                                 : getenv("SHAINET_HIP_DECODE_ROTATE")
+                                     ? (unsigned)atoi(getenv("SHAINET_HIP_DECODE_ROTATE"))
+                                     : 0x7fffffffu;
+#define SHAINET_DECODE_LAUNCH(HD_, DEV_)                                                                            \
+  SHAINET_LAUNCH_TIMED((decode_splitk_kernel<HD_, kDecodeWaves, DEV_>), grid, block, 0, stream, before, after,     \
+                       d.q_rot, d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, \
+                       sh, p.tiles_per_wg, p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev)
+  if (sh.hd == 64) {
+    if (dev)
+      SHAINET_DECODE_LAUNCH(64, true);
+    else
+      SHAINET_DECODE_LAUNCH(64, false);
+  } else {
+    if (dev)
+      SHAINET_DECODE_LAUNCH(128, true);
+    else
+      SHAINET_DECODE_LAUNCH(128, false);
+  }
+#undef SHAINET_DECODE_LAUNCH
+  return hipGetLastError();
 }
 
 }  // namespace shainet

@@ -69,8 +69,13 @@ __device__ __forceinline__ RowRef locate_row(const PrepArgs &a, const SeqTable &
 
 // Even head_dim up to 128: R head rows per wavefront, lane i < hd/2 owns the pair
 // (i, i + hd/2).  All loads of the R rows are issued before any arithmetic.
-template <int R>
-__global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st, Shape sh, int total_tokens) {
+// DEV: the sequence table is read from *dev (written by the step's plan kernel earlier on the
+// stream); a step that the plan kernel marked as skipped writes nothing.
+template <int R, bool DEV>
+__global__ __launch_bounds__(256) void prep_rows_kernel(PrepArgs a, SeqTable st_arg, Shape sh, int total_tokens,
+                                                        const DecodeDevicePlan *__restrict__ dev) {
+  if (DEV && dev->skip) return;
+  const SeqTable &st = DEV ? dev->st : st_arg;
   const int lane = threadIdx.x & 63;
   const int hd = sh.hd, half = hd >> 1;
   const int token = blockIdx.y;
@@ -310,10 +315,16 @@ __global__ void legacy_append_kernel(const float *__restrict__ staging, float *_
 }  // namespace
 
 hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, int total_tokens,
-                       hipStream_t stream) {
+                       hipStream_t stream, const DecodeDevicePlan *dev) {
   if (total_tokens <= 0) return hipSuccess;
   const int rows = sh.H + 2 * sh.KV;
   const bool fast = sh.hd <= 128 && (sh.hd & 1) == 0;
+  if (dev) {  // one row per sequence, positions known to the device only
+    if (!fast || total_tokens != st.n_seqs || total_tokens > kMaxSeqs) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((rows + 3) / 4), (unsigned)total_tokens);
+    hipLaunchKernelGGL((prep_rows_kernel<1, true>), grid, dim3(256), 0, stream, a, st, sh, total_tokens, dev);
+    return hipGetLastError();
+  }
   // few rows (decode): one row per wavefront keeps the latency short; many rows
   // (prefill): four rows per wavefront amortise the load latency
   const int rows_per_wave = fast && (long long)total_tokens * rows >= 8192 ? 4 : 1;
@@ -362,9 +373,9 @@ hipError_t launch_prep(const PrepArgs &a, const SeqTable &st, const Shape &sh, i
     if (!fast)
       hipLaunchKernelGGL(prep_rows_generic_kernel, grid, dim3(256), 0, stream, b, sub, sh, tt);
     else if (rows_per_wave == 4)
-      hipLaunchKernelGGL(prep_rows_kernel<4>, grid, dim3(256), 0, stream, b, sub, sh, tt);
+      hipLaunchKernelGGL((prep_rows_kernel<4, false>), grid, dim3(256), 0, stream, b, sub, sh, tt, nullptr);
     else
-      hipLaunchKernelGGL(prep_rows_kernel<1>, grid, dim3(256), 0, stream, b, sub, sh, tt);
+      hipLaunchKernelGGL((prep_rows_kernel<1, false>), grid, dim3(256), 0, stream, b, sub, sh, tt, nullptr);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }

@@ -74,6 +74,10 @@ _SIGNATURES = {
                                        C.c_void_p, C.c_void_p, C.c_int]),
     "shainet_attn_forward_noalloc": (C.c_int, [C.c_void_p, C.c_void_p, _i32p, _i32p, C.c_int, C.c_void_p, C.c_void_p,
                                                C.c_void_p, C.c_void_p]),
+    "shainet_kv_cache_lengths_to_device": (C.c_int, [C.c_void_p]),
+    "shainet_kv_cache_lengths_from_device": (C.c_int, [C.c_void_p]),
+    "shainet_attn_decode_step": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                           C.c_void_p]),
     "shainet_attn_last_q_rot": (C.c_int, [C.c_void_p, _f32p, C.c_int]),
     "shainet_attn_describe_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, _i32p, _i32p, _i32p]),
     "shainet_rope_apply": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_double, C.c_int]),
@@ -416,6 +420,18 @@ class AttnContext:
         _check(lib().shainet_attn_forward_noalloc(self._h, cache._h, ids, nt, n, _ptr(q), _ptr(k), _ptr(v), _ptr(out)))
         return out
 
+    def decode_step(self, cache, q, k, v, out):
+        """shainet_attn_decode_step: one new row for each of the first q.shape[0] sequences of
+        `cache`, the cached lengths read and advanced on the device (after
+        `cache.lengths_to_device()`); launches that depend on nothing but the shapes, so the call
+        can be recorded into a graph on the context's stream and replayed."""
+        n = q.shape[0]
+        assert q.is_cuda and q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and out.is_contiguous()
+        assert tuple(q.shape) == (n, self.q_dim) and tuple(k.shape) == (n, self.kv_dim)
+        assert tuple(v.shape) == tuple(k.shape) and tuple(out.shape) == tuple(q.shape)
+        _check(lib().shainet_attn_decode_step(self._h, cache._h, n, _ptr(q), _ptr(k), _ptr(v), _ptr(out)))
+        return out
+
     def prepared(self, cache, q, k, v, new_tokens, out, seq_ids=None):
         """A zero-argument callable that repeats this device-pointer forward call with nothing but
         the C call in it (tight decode loops, benchmarks): the argument checks of `forward` run
@@ -462,6 +478,14 @@ class KVCache:
 
     def len(self, seq=0):
         return lib().shainet_kv_cache_len(self._h, seq)
+
+    def lengths_to_device(self):
+        """Before `AttnContext.decode_step`: the host's lengths go to the device."""
+        _check(lib().shainet_kv_cache_lengths_to_device(self._h))
+
+    def lengths_from_device(self):
+        """After the last `decode_step` (or replay of one): waits, and takes the device's lengths back."""
+        _check(lib().shainet_kv_cache_lengths_from_device(self._h))
 
     @property
     def capacity(self):
