@@ -170,6 +170,16 @@ struct StepState {
   int cap = 0;                        // the capacity the buffers above were laid out for
 };
 
+static void release_step_state(StepState &s) {
+  if (s.d_len) (void)hipFree(s.d_len);
+  if (s.pin_len) (void)hipHostFree(s.pin_len);
+  if (s.d_plan) (void)hipFree(s.d_plan);
+  if (s.q_rot) (void)hipFree(s.q_rot);
+  if (s.partials) (void)hipFree(s.partials);
+  if (s.flags) (void)hipFree(s.flags);
+  s = StepState();
+}
+
 struct shainet_kv_cache {
   shainet_attn_ctx *ctx;
   int batch, cap;
@@ -558,12 +568,7 @@ int shainet_kv_cache_create(shainet_kv_cache **out, shainet_attn_ctx *ctx, int b
 int shainet_kv_cache_destroy(shainet_kv_cache *kc) {
   if (!kc) return SHAINET_HIP_OK;
   if (kc->ctx) (void)hipStreamSynchronize(kc->ctx->stream);
-  if (kc->step.d_len) (void)hipFree(kc->step.d_len);
-  if (kc->step.pin_len) (void)hipHostFree(kc->step.pin_len);
-  if (kc->step.d_plan) (void)hipFree(kc->step.d_plan);
-  if (kc->step.q_rot) (void)hipFree(kc->step.q_rot);
-  if (kc->step.partials) (void)hipFree(kc->step.partials);
-  if (kc->step.flags) (void)hipFree(kc->step.flags);
+  release_step_state(kc->step);
   if (kc->k) (void)hipFree(kc->k);
   if (kc->v) (void)hipFree(kc->v);
   delete kc;
@@ -887,20 +892,29 @@ extern "C" int shainet_kv_cache_lengths_to_device(shainet_kv_cache *kc) {
     return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps take caches of at most %d sequences", SHAINET_HIP_MAX_BATCH);
   StepState &st = kc->step;
   if (!st.d_len) {
+    // all of it or none: a state with some buffers missing must never reach a launch
     const DecodePlan p = step_launch_plan(c, kc->batch);
     const size_t flag_words = decode_flag_words(p);
-    HIP_TRY(hipMalloc((void **)&st.d_len, kc->batch * sizeof(int)));
-    HIP_TRY(hipHostMalloc((void **)&st.pin_len, kc->batch * sizeof(int), hipHostMallocDefault));
-    HIP_TRY(hipMalloc((void **)&st.d_plan, sizeof(DecodeDevicePlan)));
-    HIP_TRY(hipMalloc((void **)&st.q_rot, (size_t)kc->batch * c->H * c->hd * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&st.partials, decode_partial_floats(shape_of(c, kc->cap), p) * sizeof(float)));
-    HIP_TRY(hipMalloc((void **)&st.flags, flag_words * sizeof(unsigned)));
-    HIP_TRY(hipMemsetAsync(st.d_plan, 0, sizeof(DecodeDevicePlan), c->stream));
-    HIP_TRY(hipMemsetAsync(st.flags, 0, flag_words * sizeof(unsigned), c->stream));
-    if (!c->error) {
+    StepState n;
+    hipError_t e = hipMalloc((void **)&n.d_len, kc->batch * sizeof(int));
+    if (e == hipSuccess) e = hipHostMalloc((void **)&n.pin_len, kc->batch * sizeof(int), hipHostMallocDefault);
+    if (e == hipSuccess) e = hipMalloc((void **)&n.d_plan, sizeof(DecodeDevicePlan));
+    if (e == hipSuccess) e = hipMalloc((void **)&n.q_rot, (size_t)kc->batch * c->H * c->hd * sizeof(float));
+    if (e == hipSuccess)
+      e = hipMalloc((void **)&n.partials, decode_partial_floats(shape_of(c, kc->cap), p) * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc((void **)&n.flags, flag_words * sizeof(unsigned));
+    if (e == hipSuccess) e = hipMemsetAsync(n.d_plan, 0, sizeof(DecodeDevicePlan), c->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(n.flags, 0, flag_words * sizeof(unsigned), c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e == hipSuccess && !c->error) {
       c->error = c->own_error = alloc_error_word();
-      if (!c->error) return fail(SHAINET_HIP_ERR_ALLOC, "hipHostMalloc failed");
+      if (!c->error) e = hipErrorOutOfMemory;
     }
+    if (e != hipSuccess) {
+      release_step_state(n);
+      return hip_fail(e, "allocation of the decode step's buffers");
+    }
+    st = n;
   }
   // the cos/sin table must reach as far as the cache: a step cannot grow it
   if (int rc = ensure_rope_table(c, kc->cap)) return rc;

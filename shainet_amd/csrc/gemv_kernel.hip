@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
     for (int u = 0; u < 8; ++u) {
       const int row = min(k_wg + kk0 + u * RPI + sub, K - 1);
 #pragma unroll
-      for (int c = 0; c < NACC; ++c) r_first[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+      for (int c = 0; c < NACC; ++c) r_first[c][u] = __builtin_nontemporal_load((const f32x4 *)(a.w + (long long)row * ldw + c * N + col));
     }
   }
 
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
         for (int u = 0; u < 8; ++u) {
           const int row = min(k_wg + kk0 + kb + u * RPI + sub, K - 1);
 #pragma unroll
-          for (int c = 0; c < NACC; ++c) r[c][u] = *(const f32x4 *)(a.w + (long long)row * ldw + c * N + col);
+          for (int c = 0; c < NACC; ++c) r[c][u] = __builtin_nontemporal_load((const f32x4 *)(a.w + (long long)row * ldw + c * N + col));
         }
       }
 #pragma unroll
