@@ -277,6 +277,46 @@ def cpu_baseline_prefill(reps=3):
                       "path" % (n_rows, 100.0 * part / whole, reps)}
 
 
+def recorded_step(sa, torch, steps):
+    """Batch-1 decode at 4096 cached positions (Llama-3.2-1B shape) three ways, wall time per step of a
+    loop that is not waited for until its end: the host-planned call, shainet_attn_decode_step called
+    eagerly, and one such step recorded into a graph on the context's stream and replayed."""
+    H, KV, hd, L = 32, 8, 64, 4096
+    w = Workload(sa, torch, "llama1b_decode_b1_ctx4096_recorded_step", H, KV, hd, 5e5, False, [L], 1, 9)
+    n_warm = 200
+    w.alloc(4 * (steps + n_warm) + 8)
+    q, k, v, out = w.rows(1)
+    ctx, cache = w.ctx, w.cache
+    side = torch.cuda.Stream()
+    ctx.set_stream(side.cuda_stream)
+    res = {"workload": w.name}
+
+    def timed(fn, sync):
+        for _ in range(n_warm):
+            fn()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        sync()
+        return (time.perf_counter() - t0) / steps * 1e6
+
+    res["host_planned_us_per_step"] = timed(ctx.prepared(cache, q[0], k[0], v[0], [1], out), ctx.sync)
+    cache.truncate(0, L)
+    cache.lengths_to_device()
+    res["eager_step_us_per_step"] = timed(lambda: ctx.decode_step(cache, q[0], k[0], v[0], out), ctx.sync)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ctx.decode_step(cache, q[0], k[0], v[0], out)
+    with torch.cuda.stream(side):
+        res["replayed_graph_us_per_step"] = timed(graph.replay, side.synchronize)
+    cache.lengths_from_device()
+    res["cached_positions_at_end"] = cache.len(0)
+    del graph
+    w.close()
+    return res
+
+
 def layer_decode(sa, np, steps):
     """BASELINE configs[0] on the device: one Llama-3.2-1B-shaped attention layer (hidden 2048, 32 Q /
     8 KV heads, head_dim 64), projections included, 512 cached positions, one new row per call, host
@@ -508,6 +548,9 @@ def main():
 
     if want("llama1b_model_greedy_decode_ctx512"):
         results["llama1b_model_greedy_decode_ctx512"] = model_decode(sa, np, max(20, K // 4))
+
+    if want("llama1b_decode_b1_ctx4096_recorded_step"):
+        results["llama1b_decode_b1_ctx4096_recorded_step"] = recorded_step(sa, torch, max(100, K))
 
     h = results[head.name]
     line = {
