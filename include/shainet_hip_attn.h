@@ -329,6 +329,30 @@ int shainet_llama_model_cache_len(const shainet_llama_model *model);
  * them on the device (the call is then asynchronous; the sampling calls and _sync wait). */
 int shainet_llama_model_run(shainet_llama_model *model, const int *tokens, int n_tokens, float *logits);
 int shainet_llama_model_sync(shainet_llama_model *model);
+/* How a run of ONE token walks the blocks (Network#run's loop over the layers, network_run.cr:199-204,
+ * each LlamaBlock#forward_cached of llama_block.cr:189-196): one launch per product, or the whole
+ * stack as a single launch of one workgroup per compute unit with barriers between the phases of a
+ * block and the next product's first weights requested before each barrier.  The single launch
+ * needs head_dim a power of two <= 128, 1, 2, 4 or 8 query heads per kv head, d_model and ff_hidden
+ * multiples of 4 and the same geometry in every block, and must have the device's compute units to
+ * itself while it runs (its workgroups wait for each other; the wait is bounded and a give-up is
+ * reported by the next _sync / logits read as SHAINET_HIP_ERR_RUNTIME).  AUTO (the default) is one
+ * launch per product, which measured faster on the shapes tried; the variable
+ * SHAINET_HIP_PERSISTENT_STEP makes AUTO the single launch where the geometry fits.  Results of
+ * the two agree to rounding (different summation orders).  No counterpart in the reference. */
+#define SHAINET_HIP_DECODE_AUTO 0
+#define SHAINET_HIP_DECODE_PER_PRODUCT 1
+#define SHAINET_HIP_DECODE_PERSISTENT 2 /* runs of one token fail when the geometry does not fit */
+int shainet_llama_model_set_decode_mode(shainet_llama_model *model, int mode);
+/* SHAINET_HIP_DECODE_PER_PRODUCT or SHAINET_HIP_DECODE_PERSISTENT: what a run of one token uses now */
+int shainet_llama_model_decode_mode_in_use(shainet_llama_model *model);
+/* Tuning aid: with SHAINET_HIP_STEP_TRACE set before the model's first single-launch step, every
+ * workgroup of such a step records its 100 MHz clock at the launch's start and at up to 24 points
+ * of every block (the first ten: after the x slice of the q|k|v product, then before and after
+ * each of the five barriers); this copies the last step's readings, [workgroups][*per_workgroup]
+ * with *per_workgroup = 1 + 24 * layers. */
+int shainet_llama_model_step_trace(shainet_llama_model *model, long long *out, int capacity, int *workgroups,
+                                   int *per_workgroup);
 int shainet_llama_model_read_logits(shainet_llama_model *model, float *logits);
 /* replace the device logits row by host values [vocab]: lets the sampling calls run on a row that
  * was computed or edited elsewhere (the reference's Sampler takes any SimpleMatrix row) */

@@ -1027,6 +1027,13 @@ int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int n
   return SHAINET_HIP_OK;
 }
 
+// The rows shainet_attn_begin_prepared made room for are in the cache (a kernel of the caller's
+// appended them and did the attention over them): count them.
+void shainet_attn_commit_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens) {
+  kc->len[0] += new_tokens;
+  c->last_rows = 0;
+}
+
 int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out) {
   if (!c || !kc || kc->ctx != c || !out)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");

@@ -22,6 +22,7 @@
 #include "attn_kernels.hpp"
 #include "block_kernels.hpp"
 #include "llama_internal.hpp"
+#include "step_kernel.hpp"
 
 using namespace shainet;
 
@@ -344,6 +345,52 @@ int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out) 
   *out = LlamaBlockBuffers{l->w_qkv, l->w_o, b->gate_up, b->down, b->norm1, b->norm2,
                            b->d_model, l->q_dim, l->kv_dim, b->ff_hidden};
   return SHAINET_HIP_OK;
+}
+
+// One decode step of the whole stack in one launch (step_kernel.hip): where this block's weights,
+// parameters and cache are, with room for one more row made first (ensure_gpu_cache!,
+// llama_block.cr:497-520); *pos = rows cached so far.  The step's kernel appends the row;
+// shainet_llama_block_step_commit counts it afterwards.
+int shainet_llama_block_step_begin(shainet_llama_block *b, StepLayer *out, int *pos) {
+  shainet_llama_attn *l = b->attn;
+  if (!l->w_qkv || !l->w_o || !b->gate_up || !b->down) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
+  int rc = ensure_context(l);
+  if (rc) return rc;
+  const int cap = shainet_kv_cache_capacity(l->cache);
+  if (l->cache_len + 1 > cap && (rc = shainet_kv_cache_reserve(l->cache, 2 * cap))) return rc;
+  GemvPrep where;
+  if ((rc = shainet_attn_begin_prepared(l->ctx, l->cache, 1, &where))) return rc;
+  out->w_qkv = l->w_qkv;
+  out->w_o = l->w_o;
+  out->w_gu = b->gate_up;
+  out->w_down = b->down;
+  out->norm1 = b->norm1;
+  out->norm2 = b->norm2;
+  out->b_q = where.b_q;
+  out->b_k = where.b_k;
+  out->b_v = where.b_v;
+  out->q_norm = where.q_norm;
+  out->k_norm = where.k_norm;
+  out->rope_tab = where.rope_tab;
+  out->kc = where.kc;
+  out->vc = where.vc;
+  out->cap = where.cap;
+  out->pad_ = 0;
+  *pos = where.start_pos;
+  return SHAINET_HIP_OK;
+}
+void shainet_llama_block_step_commit(shainet_llama_block *b) {
+  shainet_llama_attn *l = b->attn;
+  shainet_attn_commit_prepared(l->ctx, l->cache, 1);
+  l->cache_len += 1;
+}
+// The block's geometry, for the planner of the step kernel.
+void shainet_llama_block_geometry(const shainet_llama_block *b, int *H, int *KV, int *hd, int *ff, double *qk_eps) {
+  *H = b->attn->num_heads;
+  *KV = b->attn->num_kv_heads;
+  *hd = b->attn->head_dim;
+  *ff = b->ff_hidden;
+  *qk_eps = b->attn->qk_norm_eps;
 }
 
 // Forget the cached rows past `len` (generation that ran ahead of a stop token).

@@ -22,6 +22,8 @@ struct GemvPrep;
 }
 int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, shainet::GemvPrep *where);
 int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out);
+// capi.hip: instead of finish, when the caller's own kernel appended the rows and attended over them
+void shainet_attn_commit_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens);
 // capi.hip: the pinned host word a context's kernels report a given-up wait into; a block or a
 // model that owns the context makes it the owner's word (null = back to the context's own)
 void shainet_attn_adopt_error_word(shainet_attn_ctx *c, int *word);

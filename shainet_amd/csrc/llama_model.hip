@@ -7,6 +7,10 @@
 // top-k selection of text/sampler.cr run on them without a copy of the vocab row.
 #include <hip/hip_runtime.h>
 
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
 #include <new>
 #include <string>
 #include <vector>
@@ -15,6 +19,7 @@
 #include "attn_kernels.hpp"
 #include "block_kernels.hpp"
 #include "llama_internal.hpp"
+#include "step_kernel.hpp"
 
 using namespace shainet;
 
@@ -23,6 +28,38 @@ int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, i
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream);
 int shainet_llama_block_truncate(shainet_llama_block *b, int len);
 void shainet_llama_block_share_error_word(shainet_llama_block *b, int *word);
+int shainet_llama_block_step_begin(shainet_llama_block *b, shainet::StepLayer *out, int *pos);
+void shainet_llama_block_step_commit(shainet_llama_block *b);
+void shainet_llama_block_geometry(const shainet_llama_block *b, int *H, int *KV, int *hd, int *ff, double *qk_eps);
+
+// What the one-launch decode step (step_kernel.hip) keeps between steps.
+struct ModelStep {
+  int mode = 0;          // SHAINET_HIP_DECODE_*: 0 auto, 1 one launch per product, 2 one launch per step or an error
+  bool planned = false;  // plan holds the answer for this model's geometry
+  StepPlan plan = {};
+  int n_wgs = 0;
+  int H = 0, KV = 0, hd = 0, ff = 0;
+  double qk_eps = 0.0;
+  StepLayer *d_layers = nullptr;
+  std::vector<StepLayer> layers;  // what d_layers holds
+  float *parts = nullptr;         // the five partial areas, one allocation
+  unsigned *bar = nullptr;        // the barrier's words, then as many more where the give-up test sends arrivals
+  unsigned epoch = 0;
+  bool lose_marks = false;
+  long long *trace = nullptr;     // device, [n_wgs][1 + kStepTraceSlots layers]; SHAINET_HIP_STEP_TRACE only
+  void release() {
+    if (d_layers) (void)hipFree(d_layers);
+    if (parts) (void)hipFree(parts);
+    if (bar) (void)hipFree(bar);
+    if (trace) (void)hipFree(trace);
+    d_layers = nullptr;
+    parts = nullptr;
+    bar = nullptr;
+    trace = nullptr;
+    layers.clear();
+    planned = false;
+  }
+};
 
 struct shainet_llama_model {
   int vocab = 0, d_model = 0;
@@ -46,6 +83,7 @@ struct shainet_llama_model {
   int *d_ids = nullptr;    // kMaxTopK ids, then the count
   float *d_vals = nullptr;
   int *d_gen = nullptr;    // generated ids of one chunk of shainet_llama_model_generate_greedy
+  ModelStep step;
 };
 
 namespace {
@@ -118,20 +156,142 @@ int run_topk(shainet_llama_model *m, int k, bool finite_only, int *ids, float *v
   return SHAINET_HIP_OK;
 }
 
+// Decides once per model whether its decode steps can run as one launch.
+void plan_model_step(shainet_llama_model *m) {
+  ModelStep &st = m->step;
+  st.planned = true;
+  st.plan.ok = false;
+  // AUTO: one launch per product.  Measured on the 16-block, d_model 2048 shape at 512 cached positions:
+  // 1.31 ms per token with one launch per product, 1.36 ms with the single launch (its five barriers
+  // per block and the sums of partial results after them cost what the launches did); the variable
+  // SHAINET_HIP_PERSISTENT_STEP makes AUTO take the single launch where the geometry fits.
+  static const bool auto_persistent = getenv("SHAINET_HIP_PERSISTENT_STEP") != nullptr;
+  if (st.mode == SHAINET_HIP_DECODE_PER_PRODUCT || (st.mode == SHAINET_HIP_DECODE_AUTO && !auto_persistent)) return;
+  hipDeviceProp_t prop;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
+  st.n_wgs = prop.multiProcessorCount;  // one workgroup per compute unit, all resident at once
+  if (const char *env = getenv("SHAINET_HIP_STEP_WGS")) {  // tuning knob; never more than the compute units
+    const int v = atoi(env);
+    if (v >= 1 && v < st.n_wgs) st.n_wgs = v;
+  }
+  shainet_llama_block_geometry(m->blocks[0], &st.H, &st.KV, &st.hd, &st.ff, &st.qk_eps);
+  for (shainet_llama_block *b : m->blocks) {
+    int H, KV, hd, ff;
+    double qe;
+    shainet_llama_block_geometry(b, &H, &KV, &hd, &ff, &qe);
+    if (H != st.H || KV != st.KV || hd != st.hd || ff != st.ff || qe != st.qk_eps) return;
+  }
+  const StepPlan p = plan_step(m->d_model, st.H, st.KV, st.hd, st.ff, st.n_wgs);
+  if (!p.ok) return;
+  const size_t floats = p.qkv_floats + p.attn_floats + p.o_floats + p.gu_floats + p.down_floats;
+  const size_t n_layers = m->blocks.size();
+  st.lose_marks = getenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS") != nullptr;
+  const bool want_trace = getenv("SHAINET_HIP_STEP_TRACE") != nullptr;
+  const size_t trace_bytes = (size_t)st.n_wgs * (1 + kStepTraceSlots * n_layers) * sizeof(long long);
+  if (hipMalloc((void **)&st.d_layers, n_layers * sizeof(StepLayer)) != hipSuccess ||
+      hipMalloc((void **)&st.parts, floats * sizeof(float)) != hipSuccess ||
+      hipMalloc((void **)&st.bar, 2 * step_barrier_words(st.n_wgs) * sizeof(unsigned)) != hipSuccess ||
+      hipMemset(st.bar, 0, 2 * step_barrier_words(st.n_wgs) * sizeof(unsigned)) != hipSuccess ||
+      hipMemset(st.parts, 0, floats * sizeof(float)) != hipSuccess ||
+      (want_trace && (hipMalloc((void **)&st.trace, trace_bytes) != hipSuccess ||
+                      hipMemset(st.trace, 0, trace_bytes) != hipSuccess))) {
+    (void)hipGetLastError();
+    st.release();
+    st.planned = true;
+    return;
+  }
+  st.epoch = 0;
+  st.plan = p;
+}
+
+// One new token through all blocks in one launch; m->act[0] receives the last block's output row.
+// Returns -1 when this step has to take the launch-per-product path instead.
+int run_step(shainet_llama_model *m, const int *d_token) {
+  ModelStep &st = m->step;
+  if (!st.planned) plan_model_step(m);
+  if (!st.plan.ok) return -1;
+  const size_t n_layers = m->blocks.size();
+  std::vector<StepLayer> now(n_layers);
+  int pos = -1, rc;
+  for (size_t i = 0; i < n_layers; ++i) {
+    int p = 0;
+    if ((rc = shainet_llama_block_set_stream(m->blocks[i], m->stream))) return rc;
+    if ((rc = shainet_llama_block_step_begin(m->blocks[i], &now[i], &p))) return rc;
+    if (i == 0) pos = p;
+    if (p != pos) return -1;  // blocks that were driven one by one hold different lengths
+  }
+  if (st.layers.size() != n_layers || memcmp(st.layers.data(), now.data(), n_layers * sizeof(StepLayer)) != 0) {
+    // pageable source: the copy has left `now` when the call returns; ordered on the stream
+    // behind the steps that still read the old table
+    if (hipMemcpyAsync(st.d_layers, now.data(), n_layers * sizeof(StepLayer), hipMemcpyHostToDevice, m->stream) !=
+        hipSuccess)
+      return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(layer table) failed");
+    st.layers = now;
+  }
+  const StepPlan &p = st.plan;
+  StepArgs a = {};
+  a.layers = st.d_layers;
+  a.n_layers = (int)n_layers;
+  a.d = m->d_model;
+  a.H = st.H;
+  a.KV = st.KV;
+  a.hd = st.hd;
+  a.ff = st.ff;
+  a.eps = m->eps;
+  a.qk_eps = st.qk_eps;
+  a.scale = (float)(1.0 / sqrt((double)st.hd));  // llama_block.cr:249
+  a.qkv = p.qkv;
+  a.wo = p.wo;
+  a.gu = p.gu;
+  a.down = p.down;
+  a.attn_chunks = p.attn_chunks;
+  a.attn_ck = step_keys_per_chunk(p, pos);
+  a.embedding = m->embedding;
+  a.token = d_token;
+  a.pos = pos;
+  a.x_out = m->act[0].p;
+  a.qkv_part = st.parts;
+  a.attn_part = a.qkv_part + p.qkv_floats;
+  a.o_part = a.attn_part + p.attn_floats;
+  a.gu_part = a.o_part + p.o_floats;
+  a.down_part = a.gu_part + p.gu_floats;
+  a.bar = st.bar;
+  a.bar_set = st.lose_marks ? st.bar + step_barrier_words(st.n_wgs) : st.bar;
+  a.epoch0 = st.epoch;
+  a.spin_limit = st.lose_marks ? 200 : (1 << 22);
+  a.error = m->error;
+  a.trace = st.trace;
+  const hipError_t e = launch_step(a, st.n_wgs, p.lds_bytes, m->stream);
+  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("step launch: ") + hipGetErrorString(e));
+  st.epoch += (unsigned)kStepBarriersPerLayer * (unsigned)n_layers;
+  for (shainet_llama_block *b : m->blocks) shainet_llama_block_step_commit(b);
+  return SHAINET_HIP_OK;
+}
+
 // Network#run on token ids that already sit in device memory; asynchronous.
 int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T) {
   const int d = m->d_model;
   if (!m->act[0].reserve((size_t)T * d) || !m->act[1].reserve((size_t)T * d) || !m->logits.reserve((size_t)m->vocab))
     return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   m->have_logits = false;
-  hipError_t e = launch_embed(m->embedding, d_tokens, m->act[0].p, T, d, m->stream);
-  if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
-  int cur = 0, rc;
-  for (shainet_llama_block *b : m->blocks) {
-    if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
-    if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
-    cur ^= 1;
+  int cur = 0, rc = -1;
+  if (T == 1) {
+    rc = run_step(m, d_tokens);
+    if (rc > 0) return rc;
+    if (rc < 0 && m->step.mode == SHAINET_HIP_DECODE_PERSISTENT)
+      return fail(SHAINET_HIP_ERR_ARGUMENT, "this model's geometry does not fit the one-launch decode step");
   }
+  if (rc < 0) {
+    hipError_t e = launch_embed(m->embedding, d_tokens, m->act[0].p, T, d, m->stream);
+    if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
+    for (shainet_llama_block *b : m->blocks) {
+      if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
+      if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
+      cur ^= 1;
+    }
+  }
+  hipError_t e = hipSuccess;
   // the final norm runs over every row in the reference; only the last one is used afterwards
   const float *last = m->act[cur].p + (size_t)(T - 1) * d;
   Fused fin;
@@ -187,6 +347,7 @@ int shainet_llama_model_destroy(shainet_llama_model *m) {
   if (m->d_gen) (void)hipFree(m->d_gen);
   if (m->topk_scratch) (void)hipFree(m->topk_scratch);
   m->proj.release();
+  m->step.release();
   for (DevF *f : {&m->act[0], &m->act[1], &m->logits}) f->release();
   if (m->stream) (void)hipStreamDestroy(m->stream);
   free_error_word(m->error);
@@ -312,6 +473,36 @@ int shainet_llama_model_generate_greedy(shainet_llama_model *m, int max_tokens, 
       out[(*n_out)++] = host_ids[i];
     }
   }
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_set_decode_mode(shainet_llama_model *m, int mode) {
+  if (!m) return fail(SHAINET_HIP_ERR_ARGUMENT, "model is null");
+  if (mode != SHAINET_HIP_DECODE_AUTO && mode != SHAINET_HIP_DECODE_PER_PRODUCT && mode != SHAINET_HIP_DECODE_PERSISTENT)
+    return fail(SHAINET_HIP_ERR_ARGUMENT, "mode must be one of SHAINET_HIP_DECODE_*");
+  if (m->stream && hipStreamSynchronize(m->stream) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "hipStreamSynchronize failed");
+  m->step.release();
+  m->step.mode = mode;
+  return SHAINET_HIP_OK;
+}
+
+int shainet_llama_model_decode_mode_in_use(shainet_llama_model *m) {
+  if (!m || m->blocks.empty()) return -1;
+  if (!m->step.planned) plan_model_step(m);
+  return m->step.plan.ok ? SHAINET_HIP_DECODE_PERSISTENT : SHAINET_HIP_DECODE_PER_PRODUCT;
+}
+
+int shainet_llama_model_step_trace(shainet_llama_model *m, long long *out, int capacity, int *workgroups, int *per_workgroup) {
+  if (!m || !workgroups || !per_workgroup) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
+  *workgroups = m->step.n_wgs;
+  *per_workgroup = 1 + kStepTraceSlots * (int)m->blocks.size();
+  if (!m->step.trace) return fail(SHAINET_HIP_ERR_ARGUMENT, "no trace: set SHAINET_HIP_STEP_TRACE before the model's first decode step");
+  const long long n = (long long)*workgroups * *per_workgroup;
+  if (!out || capacity < n) return fail(SHAINET_HIP_ERR_CAPACITY, "the trace holds " + std::to_string(n) + " readings");
+  if ((m->stream && hipStreamSynchronize(m->stream) != hipSuccess) ||
+      hipMemcpy(out, m->step.trace, (size_t)n * sizeof(long long), hipMemcpyDeviceToHost) != hipSuccess)
+    return fail(SHAINET_HIP_ERR_RUNTIME, "copying the trace failed");
   return SHAINET_HIP_OK;
 }
 

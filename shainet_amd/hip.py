@@ -125,6 +125,10 @@ _SIGNATURES = {
     "shainet_llama_model_cache_len": (C.c_int, [C.c_void_p]),
     "shainet_llama_model_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, _f32p]),
     "shainet_llama_model_sync": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_set_decode_mode": (C.c_int, [C.c_void_p, C.c_int]),
+    "shainet_llama_model_decode_mode_in_use": (C.c_int, [C.c_void_p]),
+    "shainet_llama_model_step_trace": (C.c_int, [C.c_void_p, C.POINTER(C.c_longlong), C.c_int, C.POINTER(C.c_int),
+                                                 C.POINTER(C.c_int)]),
     "shainet_llama_model_read_logits": (C.c_int, [C.c_void_p, _f32p]),
     "shainet_llama_model_write_logits": (C.c_int, [C.c_void_p, _f32p]),
     "shainet_llama_model_greedy": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
@@ -744,6 +748,29 @@ class LlamaModel:
 
     def sync(self):
         _check(lib().shainet_llama_model_sync(self._h))
+
+    DECODE_AUTO, DECODE_PER_PRODUCT, DECODE_PERSISTENT = 0, 1, 2
+
+    def set_decode_mode(self, mode):
+        """How a run of one token walks the blocks: one launch per product (DECODE_AUTO, the
+        default), or the whole stack in a single launch (DECODE_PERSISTENT)."""
+        _check(lib().shainet_llama_model_set_decode_mode(self._h, mode))
+
+    @property
+    def decode_mode_in_use(self):
+        return lib().shainet_llama_model_decode_mode_in_use(self._h)
+
+    def step_trace(self):
+        """Clock readings (100 MHz) of the last single-launch step, [workgroups, 1 + 24 * layers];
+        needs SHAINET_HIP_STEP_TRACE in the environment before the model's first step."""
+        import numpy as np
+
+        wgs, per = C.c_int(), C.c_int()
+        lib().shainet_llama_model_step_trace(self._h, None, 0, C.byref(wgs), C.byref(per))
+        out = np.zeros((max(wgs.value, 1), max(per.value, 1)), np.int64)
+        _check(lib().shainet_llama_model_step_trace(self._h, out.ctypes.data_as(C.POINTER(C.c_longlong)), out.size,
+                                                    C.byref(wgs), C.byref(per)))
+        return out
 
     def generate_greedy(self, max_tokens, stop_ids=()):
         """The greedy generation loop on the device, from the logits of the last `run`: returns
