@@ -36,15 +36,25 @@ def headline_lengths():
     return [int(x) for x in np.random.default_rng(2024).integers(2048, 8193, 16)]
 
 
-# name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence (None = the headline's)
-HEADLINE = ("qwen3_8b_decode_b16_ctx2048-8192", 32, 8, 128, 1e6, True, None)
+# name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence (None = the headline's), new rows per sequence
+HEADLINE = ("qwen3_8b_decode_b16_ctx2048-8192", 32, 8, 128, 1e6, True, None, 1)
+HEADLINE_MIN_SAMPLES = 100  # event-timed launches of the headline kernel, whatever --steps is
 DECODE_WORKLOADS = [
-    ("llama1b_decode_b1_ctx1024", 32, 8, 64, 5e5, False, [1024]),
-    ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096]),
-    ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384]),
-    ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4),
+    ("llama1b_decode_b1_ctx1024", 32, 8, 64, 5e5, False, [1024], 1),
+    ("llama1b_decode_b1_ctx4096", 32, 8, 64, 5e5, False, [4096], 1),
+    ("llama1b_decode_b1_ctx16384", 32, 8, 64, 5e5, False, [16384], 1),
+    ("qwen3_30b_decode_b4_ctx32768", 32, 4, 128, 1e6, True, [32768] * 4, 1),
     # the headline shape with every sequence near the top of its length range (1.07 GB per step)
-    ("qwen3_8b_decode_b16_ctx8192", 32, 8, 128, 1e6, True, [7936] * 16),
+    ("qwen3_8b_decode_b16_ctx8192", 32, 8, 128, 1e6, True, [7936] * 16, 1),
+    # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
+    # through the split-K decode kernel as further columns of its tiles: the same bytes, HBM bound)
+    ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, None, 4),
+    # not BASELINE configurations: head dims without an MFMA instantiation (one wavefront per row and
+    # head, llama_block.cr:80-89 accepts any head_dim) and 32 query heads per kv head (more columns
+    # than the decode kernel's tile: the MFMA prefill kernel serves it), to put a number on both
+    ("generic_hd96_decode_b1_ctx4096", 32, 8, 96, 5e5, False, [4096], 1),
+    ("generic_hd256_decode_b1_ctx4096", 16, 4, 256, 5e5, False, [4096], 1),
+    ("mqa_g32_hd128_decode_b1_ctx4096", 32, 1, 128, 5e5, False, [4096], 1),
 ]
 # name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence, new rows per sequence
 PREFILL_WORKLOADS = [
@@ -53,9 +63,6 @@ PREFILL_WORKLOADS = [
     ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512),
     # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
     ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048),
-    # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
-    # through the split-K decode kernel as further columns of its tiles)
-    ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, None, 4),
 ]
 
 
@@ -105,12 +112,14 @@ class Workload:
         torch.cuda.synchronize()
         return q, k, v, out
 
-    def run_decode(self, steps, warmup):
-        """Consecutive decode steps appending to the cache."""
-        torch, ctx = self.torch, self.ctx
-        self.alloc(2 * steps + 1)
+    def run_decode(self, steps, warmup, min_samples=0):
+        """Consecutive decode steps (self.T new rows per sequence) appending to the cache; the kernel is
+        then timed with events over max(steps, min_samples) further steps."""
+        torch, ctx, T = self.torch, self.ctx, self.T
+        prof_steps = max(steps, min_samples)
+        self.alloc(T * (steps + prof_steps) + 1)
         q, k, v, out = self.rows(min(2 * steps, 64))
-        nt = [1] * self.B
+        nt = [T] * self.B
         n = q.shape[0]
         # the timed loop holds nothing but the C call: the row sets are bound beforehand
         calls = [ctx.prepared(self.cache, q[i], k[i], v[i], nt, out) for i in range(n)]
@@ -148,15 +157,15 @@ class Workload:
         wall = time.perf_counter() - t0
         # second pass with HIP events around the split-K kernel only
         ctx.profile(True)
-        for i in range(steps):
+        for i in range(prof_steps):
             step(steps + i)
-        samples = ctx.profile_samples(steps + 8)
+        samples = ctx.profile_samples(prof_steps + 8)
         k_ms, launches = float(samples.sum()), len(samples)
         ctx.profile(False)
-        vis_wall = [[L + i + 1 for L in self.lens] for i in range(steps)]
-        vis_prof = [[L + steps + i + 1 for L in self.lens] for i in range(steps)]
+        vis_wall = [[L + T * (i + 1) for L in self.lens] for i in range(steps)]
+        vis_prof = [[L + T * (steps + i + 1) for L in self.lens] for i in range(prof_steps)]
         b_wall = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_wall) / steps
-        b_prof = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_prof) / steps
+        b_prof = sum(decode_bytes(self.KV, self.hd, v_) for v_ in vis_prof) / prof_steps
         us = wall / steps * 1e6
         kus = k_ms / max(launches, 1) * 1e3
         import numpy as np
@@ -360,7 +369,7 @@ def model_decode(sa, np, steps, ctx_len=512):
         b.set_ffn(*ws[4:])
     del ws
     weight_bytes = 4 * (L * (2 * d * H * hd + 2 * d * KV * hd + 3 * d * ff) + d * V)
-    # prefill of the context: more than 16 rows go through the library GEMM and the MFMA attention kernel
+    # prefill of the context: more than 16 rows go through the library's own MFMA product and the MFMA attention kernel
     prompt = list(r.integers(0, V, ctx_len))
     m.run(prompt, want_logits=False)
     m.sync()
@@ -381,8 +390,17 @@ def model_decode(sa, np, steps, ctx_len=512):
     t0 = time.perf_counter()
     n = len(m.generate_greedy(steps))
     dt = (time.perf_counter() - t0) / max(n, 1)
+    # the same steps as one launch per token (the opt-in decode mode), from the same cached context
+    m.set_decode_mode(m.DECODE_PERSISTENT)
+    m.clear_cache()
+    m.run(prompt, want_logits=False)
+    m.generate_greedy(16)
+    t0 = time.perf_counter()
+    n1 = len(m.generate_greedy(steps))
+    dt1 = (time.perf_counter() - t0) / max(n1, 1)
     m.close()
     return {"workload": "llama1b_model_greedy_decode_ctx%d" % ctx_len, "us_per_token": dt * 1e6,
+            "us_per_token_single_launch_step": dt1 * 1e6,
             "tokens_per_s": 1.0 / dt, "weight_bytes_per_token": weight_bytes,
             "weight_gbps": weight_bytes / dt / 1e9, "frac_of_hbm_peak": weight_bytes / dt / 1e9 / HBM_PEAK_GBPS,
             "prefill_tokens": ctx_len, "prefill_ms": prefill_s * 1e3, "prefill_tokens_per_s": ctx_len / prefill_s,
@@ -450,6 +468,12 @@ def yardsticks(torch, reps=5):
         torch.cuda.synchronize()
         out[key] = round(amount() / (e0.elapsed_time(e1) / reps * 1e3), 1)
     del a
+    # what a launch costs with no work in it, by the kernels' own clocks: one empty kernel of 256
+    # workgroups, and two of them one after the other on one stream (one kernel boundary: the floor
+    # under a step that is a prep kernel followed by an attention kernel)
+    out["launch_us"] = round(hip.launch_latency(1, 200, 256, stream), 2)
+    out["launch_pair_us"] = round(hip.launch_latency(2, 200, 256, stream), 2)
+    out["launch_chain8_us"] = round(hip.launch_latency(8, 100, 256, stream), 2)
     return out
 
 
@@ -517,9 +541,9 @@ def main():
         return not only or name in only
 
     # headline: configs[2]
-    name, H, KV, hd, th, norm, _ = HEADLINE
-    head = Workload(sa, torch, name, H, KV, hd, th, norm, lens3, 1, 3)
-    results[head.name] = head.run_decode(K, W)
+    name, H, KV, hd, th, norm, _, T1 = HEADLINE
+    head = Workload(sa, torch, name, H, KV, hd, th, norm, lens3, T1, 3)
+    results[head.name] = head.run_decode(K, W, HEADLINE_MIN_SAMPLES)
     cpu = None
     if not args.no_cpu:
         cpu_us = cpu_baseline(head, 21)
@@ -529,14 +553,14 @@ def main():
                "host_cores_visible": os.cpu_count()}
     head.close()
 
-    for name, H, KV, hd, th, norm, lens in DECODE_WORKLOADS:
+    for name, H, KV, hd, th, norm, lens, T in DECODE_WORKLOADS:
         if want(name):
-            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, 1, 5)
+            lens = lens3 if lens is None else lens
+            w = Workload(sa, torch, name, H, KV, hd, th, norm, lens, T, 5)
             results[name] = w.run_decode(K if len(lens) < 16 else max(20, K // 2), W)
             w.close()
     fewer = {"llama1b_prefill_t2048": K, "llama1b_prefill_t8192": max(5, K // 20),
-             "qwen3_30b_chunked_prefill_t512_on_16384": max(5, K // 10), "qwen3_8b_prefill_t2048": max(5, K // 2),
-             "qwen3_8b_decode_b16_4rows_ctx2048-8192": max(10, K // 4)}
+             "qwen3_30b_chunked_prefill_t512_on_16384": max(5, K // 10), "qwen3_8b_prefill_t2048": max(5, K // 2)}
     for name, H, KV, hd, th, norm, lens, T in PREFILL_WORKLOADS:
         if want(name):
             w = Workload(sa, torch, name, H, KV, hd, th, norm, lens3 if lens is None else lens, T, 7)
@@ -571,7 +595,8 @@ def main():
         "hbm_gbps": round(h["step_gbps"], 1),
         "roofline": {"bound": "hbm", "kernel": ROOFLINE_KERNELS["roofline"][0], "achieved": round(h["kernel_gbps"], 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(h["kernel_gbps"] / HBM_PEAK_GBPS, 4),
-                     "kernel_us": round(h["kernel_us"], 2), "kernel_us_p10_p50_p90": [round(h["kernel_us_p10"], 2),
+                     "kernel_us": round(h["kernel_us"], 2), "kernel_samples": h["launches"],
+                     "kernel_us_p10_p50_p90": [round(h["kernel_us_p10"], 2),
                                                                                       round(h["kernel_us_p50"], 2),
                                                                                       round(h["kernel_us_p90"], 2)],
                      "bytes_per_launch": int(h["kernel_bytes"]),
@@ -595,8 +620,13 @@ def main():
                                     "traffic": load_traffic(ROOFLINE_KERNELS["roofline_prefill"][0], p["workload"])}
     if p and not args.no_cpu:
         line["cpu_baseline_prefill"] = cpu_baseline_prefill()
-    if not args.only:
-        line["yardsticks"] = yardsticks(torch)
+    yard = yardsticks(torch)
+    line["yardsticks"] = yard
+    # every HBM-bound figure also as a fraction of what a plain read of 1 GiB reaches on this box
+    for r in list(line["workloads"].values()) + [line["roofline"]]:
+        f = r.get("frac_of_hbm_peak", r.get("frac") if r is line["roofline"] else None)
+        if f is not None:
+            r["frac_of_stream_yardstick"] = round(f * HBM_PEAK_GBPS / yard["stream_read_gbps"], 4)
     print(json.dumps(line))
 
 

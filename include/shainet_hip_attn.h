@@ -164,7 +164,12 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
  * (the calls the split-K decode kernel takes); every position below the max_positions the
  * context was created with; sizes within the array.  All calls on one GPU share the array:
  * two calls of this entry point that overlap in time on one GPU (different contexts on
- * different streams) race; calls on one context, or one after the other, do not. */
+ * different streams) race; calls on one context, or one after the other, do not.
+ * The address of the array on a device is looked up when a context is created on it, not in the
+ * call.  Under stream capture the call may be recorded, but the recording is good for one run
+ * only: the launch is planned on the host (start positions and spans are kernel arguments, the
+ * cache length advances once, when the call is made), so a replay would write the same cache row
+ * again.  shainet_attn_decode_step is the entry point whose recording can be replayed. */
 int shainet_attn_forward_noalloc(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const int *seq_ids,
                                  const int *new_tokens, int n_seqs, const float *q, const float *k, const float *v,
                                  float *out);
@@ -189,7 +194,10 @@ int shainet_attn_forward_noalloc(shainet_attn_ctx *ctx, shainet_kv_cache *cache,
  *   (or shainet_attn_sync) then returns SHAINET_HIP_ERR_CAPACITY.
  * shainet_kv_cache_lengths_from_device: waits for the stream and copies the device's lengths
  *   back, so that shainet_kv_cache_len and the other entry points see the rows the steps appended.
- * Between the two copies the host's lengths are stale: use no other entry point on the cache.
+ * Between the two copies the host's lengths are stale: every other entry point that reads or writes
+ * them (shainet_attn_forward and its variants, fill, clear, truncate, reserve, a second
+ * lengths_to_device) is refused with SHAINET_HIP_ERR_ARGUMENT and shainet_kv_cache_len returns -1;
+ * after lengths_from_device a step needs lengths_to_device again.
  * A recorded step holds the addresses of the cache, of the context's cos/sin table, bias and
  * QK-norm weights: record it again after shainet_kv_cache_reserve, shainet_attn_set_bias, or a
  * call on another cache of the same context that reaches beyond the table's positions. */
@@ -263,8 +271,11 @@ int shainet_llama_attn_forward_full(shainet_llama_attn *layer, const float *x, i
  * dispatches (llama_block.cr:726-768: SimpleMatrix#* on the host, cuBLAS SGEMM on the device,
  * cuda.cr:237-247): up to 16 rows run the split GEMV of the decode step, more rows the MFMA
  * kernel of the prefill.  fp32 accumulation (the host path of the reference accumulates in
- * fp64, simple_matrix.cr:61-74).  The handle-less calls share one grow-only scratch buffer:
- * one caller at a time. */
+ * fp64, simple_matrix.cr:61-74).  The handle-less calls keep one grow-only scratch set per stream
+ * (partial products of split shapes and their flag words): calls on different streams may overlap,
+ * calls on one stream are ordered by it; one host thread at a time inside the call.  A kernel of
+ * an earlier call on the same stream that gave up its bounded wait for partial sums is reported by
+ * the next call on that stream (SHAINET_HIP_ERR_RUNTIME), which then does nothing else. */
 int shainet_hip_matmul_f32(const float *x, long long x_stride, const float *w, const float *res, float *y, int rows,
                            int k, int n, void *stream);
 
@@ -328,6 +339,11 @@ int shainet_llama_model_cache_len(const shainet_llama_model *model);
 /* tokens: host ids [n_tokens], appended to every block's cache.  logits: host [vocab], or null to leave
  * them on the device (the call is then asynchronous; the sampling calls and _sync wait). */
 int shainet_llama_model_run(shainet_llama_model *model, const int *tokens, int n_tokens, float *logits);
+/* The same with the network's use_kv_cache switched off (network_setup.cr:32, network_run.cr:199-204:
+ * LlamaBlock#forward instead of forward_cached in every block): the n_tokens rows attend among
+ * themselves from position 0, every block's cache and cache length stay as they are.  The logits of
+ * the last row are left for the sampling calls like those of shainet_llama_model_run. */
+int shainet_llama_model_run_full(shainet_llama_model *model, const int *tokens, int n_tokens, float *logits);
 int shainet_llama_model_sync(shainet_llama_model *model);
 /* How a run of ONE token walks the blocks (Network#run's loop over the layers, network_run.cr:199-204,
  * each LlamaBlock#forward_cached of llama_block.cr:189-196): one launch per product, or the whole
@@ -449,6 +465,15 @@ int shainet_hip_stream_read_f32(const float *src, float *sink, long long n, int 
  * the clock the device holds under that load, the yardstick next to the published peak for
  * the prefill kernels.  No counterpart in the reference. */
 int shainet_hip_mfma_f32_loop(float *sink, int iters, int workgroups, long long *flops, void *stream);
+
+/* What a launch costs on the device with no work in it: `chain` kernels of `workgroups` empty
+ * workgroups, one after the other on `stream`, timed from the first kernel's own first clock
+ * reading to the last kernel's last one (hipExtLaunchKernel events, as the attention kernels are
+ * timed); *us = the median of `reps` such chains, in microseconds.  chain = 1 is the shortest
+ * kernel the device runs, chain = 2 adds one kernel boundary: the floor under every step that
+ * is a prep kernel followed by an attention kernel.  Waits for the stream.  No counterpart in the
+ * reference. */
+int shainet_hip_launch_latency(int chain, int reps, int workgroups, float *us, void *stream);
 
 #ifdef __cplusplus
 }

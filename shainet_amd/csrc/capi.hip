@@ -64,6 +64,8 @@ int check_error_word(int *w) {
 
 namespace {
 
+int scratch_on_current_device(unsigned char **out);  // below, with the static scratch of the entry point that allocates nothing
+
 int hip_fail(hipError_t e, const char *what) {
   return fail(e == hipErrorOutOfMemory ? SHAINET_HIP_ERR_ALLOC : SHAINET_HIP_ERR_RUNTIME, "%s: %s", what,
               hipGetErrorString(e));
@@ -168,6 +170,9 @@ struct StepState {
   float *partials = nullptr;          // device_plan_slots(batch, KV) slots of g columns
   unsigned *flags = nullptr;          // zero between launches
   int cap = 0;                        // the capacity the buffers above were laid out for
+  // Between shainet_kv_cache_lengths_to_device and _from_device the device's lengths are the ones that count
+  // (decode steps advance only those): every entry point that reads or writes the host's copy is refused.
+  bool lengths_on_device = false;
 };
 
 static void release_step_state(StepState &s) {
@@ -187,6 +192,15 @@ struct shainet_kv_cache {
   std::vector<int> len;
   StepState step;
 };
+
+namespace {
+int refuse_while_lengths_on_device(const shainet_kv_cache *kc, const char *what) {
+  if (!kc->step.lengths_on_device) return SHAINET_HIP_OK;
+  return fail(SHAINET_HIP_ERR_ARGUMENT,
+              "%s: the cached lengths are on the device (shainet_kv_cache_lengths_to_device); call "
+              "shainet_kv_cache_lengths_from_device first", what);
+}
+}  // namespace
 
 namespace {
 
@@ -366,7 +380,11 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
 // they share one grow-only scratch set, as the reference's class-level scratch
 // does (llama_block.cr:57-68).
 shainet_attn_ctx *legacy_ctx() {
-  static shainet_attn_ctx *c = new (std::nothrow) shainet_attn_ctx();
+  static shainet_attn_ctx *c = [] {
+    shainet_attn_ctx *n = new (std::nothrow) shainet_attn_ctx();
+    if (n) n->test_lose_marks = getenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS") != nullptr;
+    return n;
+  }();
   return c;
 }
 
@@ -411,6 +429,10 @@ void attention_kv_f32(const float *q, const float *kc, const float *vc, float *o
     fprintf(stderr, "HIP Error in attention_kv_f32: invalid arguments\n");
     return;
   }
+  // The calls are asynchronous and return nothing: what an earlier call's kernel reported (a given-up
+  // wait for partial results) is said here, the way the reference prints the launch error of every
+  // call (cuda_kernels.cu:821-824).
+  if (check_error_word(c->error)) fprintf(stderr, "HIP Error in attention_kv_f32 (an earlier call): %s\n", g_err);
   c->H = num_heads;
   c->KV = num_heads / heads_per_kv;
   c->g = heads_per_kv;
@@ -470,6 +492,10 @@ int shainet_attn_create(shainet_attn_ctx **out, int num_heads, int num_kv_heads,
   if (!rc) rc = upload(&c->d_q_norm, q_norm, head_dim);
   if (!rc) rc = upload(&c->d_k_norm, k_norm, head_dim);
   if (!rc) rc = ensure_rope_table(c, max_positions > 0 ? max_positions : 1024);
+  // the address of the static scratch of shainet_attn_forward_noalloc on this device: asked for here,
+  // once per device, so that the call itself (which may run under stream capture) only looks it up
+  unsigned char *scratch_base = nullptr;
+  if (!rc) rc = scratch_on_current_device(&scratch_base);
   if (rc) {
     shainet_attn_destroy(c);
     return rc;
@@ -577,6 +603,7 @@ int shainet_kv_cache_destroy(shainet_kv_cache *kc) {
 
 int shainet_kv_cache_clear(shainet_kv_cache *kc, int seq) {
   if (!kc || seq >= kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid sequence");
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_kv_cache_clear")) return rc;
   if (seq < 0)
     kc->len.assign(kc->batch, 0);
   else
@@ -586,6 +613,7 @@ int shainet_kv_cache_clear(shainet_kv_cache *kc, int seq) {
 
 int shainet_kv_cache_truncate(shainet_kv_cache *kc, int seq, int len) {
   if (!kc || seq < 0 || seq >= kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid sequence");
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_kv_cache_truncate")) return rc;
   if (len < 0 || len > kc->len[seq])
     return fail(SHAINET_HIP_ERR_ARGUMENT, "truncate to %d outside 0..%d", len, kc->len[seq]);
   kc->len[seq] = len;
@@ -594,6 +622,7 @@ int shainet_kv_cache_truncate(shainet_kv_cache *kc, int seq, int len) {
 
 int shainet_kv_cache_len(const shainet_kv_cache *kc, int seq) {
   if (!kc || seq < 0 || seq >= kc->batch) return -1;
+  if (refuse_while_lengths_on_device(kc, "shainet_kv_cache_len")) return -1;
   return kc->len[seq];
 }
 
@@ -605,6 +634,7 @@ float *shainet_kv_cache_v(shainet_kv_cache *kc) { return kc ? kc->v : nullptr; }
 int shainet_kv_cache_reserve(shainet_kv_cache *kc, int capacity) {
   if (!kc) return fail(SHAINET_HIP_ERR_ARGUMENT, "cache is null");
   if (capacity <= kc->cap) return SHAINET_HIP_OK;
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_kv_cache_reserve")) return rc;  // growth copies len rows
   shainet_attn_ctx *c = kc->ctx;
   const size_t row = (size_t)c->hd * sizeof(float);
   const size_t bytes = (size_t)kc->batch * c->KV * capacity * row;
@@ -637,6 +667,7 @@ int shainet_kv_cache_reserve(shainet_kv_cache *kc, int capacity) {
 int shainet_kv_cache_fill(shainet_kv_cache *kc, int seq, const float *k_rows, const float *v_rows, int n, int mem) {
   if (!kc || seq < 0 || seq >= kc->batch || n < 0 || !k_rows || !v_rows)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid fill arguments");
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_kv_cache_fill")) return rc;
   if (n > kc->cap) return fail(SHAINET_HIP_ERR_CAPACITY, "fill of %d rows exceeds capacity %d", n, kc->cap);
   shainet_attn_ctx *c = kc->ctx;
   const size_t row = (size_t)c->hd * sizeof(float);
@@ -698,6 +729,7 @@ int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, 
                  const float *q, const float *k, const float *v, long long q_stride, long long k_stride,
                  long long v_stride, float *out, int mem, const Workspace *ws) {
   if (!c || !kc || kc->ctx != c) return fail(SHAINET_HIP_ERR_ARGUMENT, "context and cache do not belong together");
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_attn_forward")) return rc;
   if (ws && mem != SHAINET_HIP_MEM_DEVICE)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "the entry point that allocates nothing takes device pointers only");
   if (!new_tokens || !q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
@@ -762,9 +794,13 @@ int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, 
     memcpy(pq, q, q_floats * sizeof(float));
     memcpy(pk, k, kv_floats * sizeof(float));
     memcpy(pv, v, kv_floats * sizeof(float));
-    HIP_TRY(hipMemcpyAsync(c->in_q.p, pq, q_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
-    HIP_TRY(hipMemcpyAsync(c->in_k.p, pk, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
-    HIP_TRY(hipMemcpyAsync(c->in_v.p, pv, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    hipError_t ce = hipMemcpyAsync(c->in_q.p, pq, q_floats * sizeof(float), hipMemcpyHostToDevice, c->stream);
+    if (ce == hipSuccess) ce = hipMemcpyAsync(c->in_k.p, pk, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream);
+    if (ce == hipSuccess) ce = hipMemcpyAsync(c->in_v.p, pv, kv_floats * sizeof(float), hipMemcpyHostToDevice, c->stream);
+    if (ce != hipSuccess) {
+      (void)hipStreamSynchronize(c->stream);  // a copy already queued may still read the staging buffer
+      return hip_fail(ce, "hipMemcpyAsync(q, k, v)");
+    }
     dq = c->in_q.p;
     dk = c->in_k.p;
     dv = c->in_v.p;
@@ -792,13 +828,19 @@ int forward_core(shainet_attn_ctx *c, shainet_kv_cache *kc, const int *seq_ids, 
   pa.kc = kc->k;
   pa.vc = kc->v;
   rc = run_attention(c, q_rot, kc->k, kc->v, dout, st, sh, rows, c->scale, c->stream, &pa, ws);
-  if (rc) return rc;  // the cached lengths stay as they were: the call did not happen
+  if (rc) {
+    // the copies out of the pinned staging buffer may still run: the next call overwrites it
+    if (mem == SHAINET_HIP_MEM_HOST) (void)hipStreamSynchronize(c->stream);
+    return rc;  // the cached lengths stay as they were: the call did not happen
+  }
   // the rows are in the cache once this call's kernels have run: @cache_len = total_len (llama_block.cr:288-289)
   for (int s = 0; s < n_seqs; ++s) kc->len[st.slot[s]] += st.n_new[s];
   c->last_rows = ws ? 0 : rows;  // shainet_attn_last_q_rot reads the context's own buffer
   if (mem == SHAINET_HIP_MEM_HOST) {
-    HIP_TRY(hipMemcpyAsync(c->pin_out.p, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream));
-    HIP_TRY(hipStreamSynchronize(c->stream));
+    const hipError_t ce = hipMemcpyAsync(c->pin_out.p, dout, q_floats * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+    const hipError_t se = hipStreamSynchronize(c->stream);  // also when the copy could not be queued
+    if (ce != hipSuccess) return hip_fail(ce, "hipMemcpyAsync(out)");
+    if (se != hipSuccess) return hip_fail(se, "hipStreamSynchronize");
     memcpy(out, c->pin_out.p, q_floats * sizeof(float));
     return check_error_word(c->error);
   }
@@ -891,6 +933,7 @@ extern "C" int shainet_kv_cache_lengths_to_device(shainet_kv_cache *kc) {
   if (kc->batch > SHAINET_HIP_MAX_BATCH)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps take caches of at most %d sequences", SHAINET_HIP_MAX_BATCH);
   StepState &st = kc->step;
+  if (int rc = refuse_while_lengths_on_device(kc, "shainet_kv_cache_lengths_to_device")) return rc;
   if (!st.d_len) {
     // all of it or none: a state with some buffers missing must never reach a launch
     const DecodePlan p = step_launch_plan(c, kc->batch);
@@ -922,6 +965,7 @@ extern "C" int shainet_kv_cache_lengths_to_device(shainet_kv_cache *kc) {
   HIP_TRY(hipMemcpyAsync(st.d_len, st.pin_len, kc->batch * sizeof(int), hipMemcpyHostToDevice, c->stream));
   HIP_TRY(hipStreamSynchronize(c->stream));
   st.cap = kc->cap;
+  st.lengths_on_device = true;
   return SHAINET_HIP_OK;
 }
 
@@ -938,6 +982,7 @@ extern "C" int shainet_kv_cache_lengths_from_device(shainet_kv_cache *kc) {
                   st.pin_len[s], s, kc->cap);
     kc->len[s] = st.pin_len[s];
   }
+  st.lengths_on_device = false;
   return check_error_word(c->error);
 }
 
@@ -947,8 +992,10 @@ extern "C" int shainet_attn_decode_step(shainet_attn_ctx *c, shainet_kv_cache *k
   if (!q || !k || !v || !out) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (n_seqs < 1 || n_seqs > kc->batch) return fail(SHAINET_HIP_ERR_ARGUMENT, "n_seqs must be in 1..%d", kc->batch);
   StepState &ss = kc->step;
-  if (!ss.d_len) return fail(SHAINET_HIP_ERR_ARGUMENT, "shainet_kv_cache_lengths_to_device has not been called");
-  if (ss.cap != kc->cap)
+  if (!ss.d_len || !ss.lengths_on_device)
+    return fail(SHAINET_HIP_ERR_ARGUMENT,
+                "shainet_kv_cache_lengths_to_device has not been called (again) since the lengths last came back to the host");
+  if (ss.cap != kc->cap)  // cannot happen while the lengths are on the device: reserve is refused then
     return fail(SHAINET_HIP_ERR_ARGUMENT, "the cache has grown since shainet_kv_cache_lengths_to_device: call it again");
   const Shape sh = shape_of(c, kc->cap);
   hipError_t e = launch_decode_plan(ss.d_len, n_seqs, sh, c->rope_positions, ss.d_plan, c->error, c->stream);

@@ -570,7 +570,7 @@ __global__ __launch_bounds__(64) void decode_plan_kernel(int *__restrict__ lens,
       out->total_tiles = 0;
       out->skip = 1;
       spans_from_shares(shares.v, 0, out->spans);  // all zero: no workgroup finds tiles
-      *error = 2;
+      if (*error == 0) *error = 2;  // a pending 1 (a given-up wait) is the graver report and stays
     }
     return;
   }

@@ -233,13 +233,15 @@ __global__ __launch_bounds__(256) void sgemm_reduce_kernel(const float *__restri
 __global__ __launch_bounds__(256) void sgemm_plain_kernel(const float *__restrict__ x, long long xs,
                                                           const float *__restrict__ w, float *__restrict__ y,
                                                           const float *__restrict__ res, int T, int K, int N) {
-  const int n = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
-  const float *xr = x + (long long)t * xs;
-  float acc = 0.f;
-  for (int k = 0; k < K; ++k) acc += xr[k] * w[(long long)k * N + n];
-  const long long o = (long long)t * N + n;
-  y[o] = res ? res[o] + acc : acc;
+  for (int t = blockIdx.y; t < T; t += gridDim.y) {  // the grid's second dimension ends at 65535
+    const float *xr = x + (long long)t * xs;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) acc += xr[k] * w[(long long)k * N + n];
+    const long long o = (long long)t * N + n;
+    y[o] = res ? res[o] + acc : acc;
+  }
 }
 
 }  // namespace
@@ -280,7 +282,7 @@ hipError_t launch_gemm(const float *x, long long x_stride, const float *w, float
   if (!x || !w || !y || T < 1 || K < 1 || N < 1 || x_stride < K) return hipErrorInvalidValue;
   const bool aligned = !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)res) & 15);
   if (!p.mfma || !aligned) {
-    hipLaunchKernelGGL(sgemm_plain_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)T), dim3(256), 0, stream, x,
+    hipLaunchKernelGGL(sgemm_plain_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)(T < 65535 ? T : 65535)), dim3(256), 0, stream, x,
                        x_stride, w, y, res, T, K, N);
     return hipGetLastError();
   }

@@ -267,7 +267,10 @@ static int attn_forward_host(shainet_llama_attn *l, const float *x, int new_toke
   memcpy(l->x_pin.p, x, xd * sizeof(float));  // the last call's copies are done: every host-pointer call ends with a wait
   if (hipMemcpyAsync(l->x.p, l->x_pin.p, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
-  if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p, Fused(), nullptr, no_cache))) return rc;
+  if ((rc = attn_forward_device(l, l->x.p, new_tokens, l->out.p, Fused(), nullptr, no_cache))) {
+    (void)hipStreamSynchronize(stream);  // the copy out of the pinned staging buffer may still run
+    return rc;
+  }
   if (hipMemcpyAsync(l->out_pin.p, l->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");
@@ -325,8 +328,8 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
 }  // namespace
 
 // used by the model (llama_model.hip)
-int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out) {
-  return block_forward_device(b, x, T, out);
+int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out, bool no_cache) {
+  return block_forward_device(b, x, T, out, no_cache);
 }
 int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out) {
   shainet_llama_attn *l = b->attn;
@@ -515,7 +518,10 @@ static int block_forward_any(shainet_llama_block *b, const float *x, int new_tok
   memcpy(b->x_pin.p, x, xd * sizeof(float));
   if (hipMemcpyAsync(b->x.p, b->x_pin.p, xd * sizeof(float), hipMemcpyHostToDevice, stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(x) failed");
-  if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p, no_cache))) return rc;
+  if ((rc = block_forward_device(b, b->x.p, new_tokens, b->out.p, no_cache))) {
+    (void)hipStreamSynchronize(stream);  // the copy out of the pinned staging buffer may still run
+    return rc;
+  }
   if (hipMemcpyAsync(b->out_pin.p, b->out.p, xd * sizeof(float), hipMemcpyDeviceToHost, stream) != hipSuccess ||
       hipStreamSynchronize(stream) != hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "copying the result back failed");

@@ -24,7 +24,7 @@
 using namespace shainet;
 
 // llama_block.hip
-int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out);
+int shainet_llama_block_forward_device(shainet_llama_block *b, const float *x, int T, float *out, bool no_cache);
 int shainet_llama_block_set_stream(shainet_llama_block *b, hipStream_t stream);
 int shainet_llama_block_truncate(shainet_llama_block *b, int len);
 void shainet_llama_block_share_error_word(shainet_llama_block *b, int *word);
@@ -269,14 +269,16 @@ int run_step(shainet_llama_model *m, const int *d_token) {
   return SHAINET_HIP_OK;
 }
 
-// Network#run on token ids that already sit in device memory; asynchronous.
-int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T) {
+// Network#run on token ids that already sit in device memory; asynchronous.  no_cache: every block's
+// LlamaBlock#forward instead of forward_cached (network_run.cr:199-204 with use_kv_cache off): the
+// rows attend among themselves from position 0 and the caches stay as they are.
+int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T, bool no_cache = false) {
   const int d = m->d_model;
   if (!m->act[0].reserve((size_t)T * d) || !m->act[1].reserve((size_t)T * d) || !m->logits.reserve((size_t)m->vocab))
     return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   m->have_logits = false;
   int cur = 0, rc = -1;
-  if (T == 1) {
+  if (T == 1 && !no_cache) {
     rc = run_step(m, d_tokens);
     if (rc > 0) return rc;
     if (rc < 0 && m->step.mode == SHAINET_HIP_DECODE_PERSISTENT)
@@ -287,7 +289,7 @@ int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T) {
     if (e != hipSuccess) return fail(SHAINET_HIP_ERR_RUNTIME, std::string("embedding launch: ") + hipGetErrorString(e));
     for (shainet_llama_block *b : m->blocks) {
       if ((rc = shainet_llama_block_set_stream(b, m->stream))) return rc;
-      if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p))) return rc;
+      if ((rc = shainet_llama_block_forward_device(b, m->act[cur].p, T, m->act[cur ^ 1].p, no_cache))) return rc;
       cur ^= 1;
     }
   }
@@ -400,7 +402,17 @@ int shainet_llama_model_cache_len(const shainet_llama_model *m) {
   return m && !m->blocks.empty() ? shainet_llama_block_cache_len(m->blocks[0]) : -1;
 }
 
+static int model_run(shainet_llama_model *m, const int *tokens, int n_tokens, float *logits, bool no_cache);
+
 int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tokens, float *logits) {
+  return model_run(m, tokens, n_tokens, logits, false);
+}
+
+int shainet_llama_model_run_full(shainet_llama_model *m, const int *tokens, int n_tokens, float *logits) {
+  return model_run(m, tokens, n_tokens, logits, true);
+}
+
+static int model_run(shainet_llama_model *m, const int *tokens, int n_tokens, float *logits, bool no_cache) {
   if (!m || !tokens || n_tokens < 1) return fail(SHAINET_HIP_ERR_ARGUMENT, "invalid arguments");
   if (!m->embedding || !m->lm_head) return fail(SHAINET_HIP_ERR_ARGUMENT, "embedding or lm_head not set");
   for (int i = 0; i < n_tokens; ++i)  // an id outside the table raises IndexError in the reference
@@ -414,7 +426,7 @@ int shainet_llama_model_run(shainet_llama_model *m, const int *tokens, int n_tok
   if (hipMemcpyAsync(m->d_tokens, tokens, (size_t)n_tokens * sizeof(int), hipMemcpyHostToDevice, m->stream) !=
       hipSuccess)
     return fail(SHAINET_HIP_ERR_RUNTIME, "hipMemcpyAsync(tokens) failed");
-  if ((rc = run_device_tokens(m, m->d_tokens, n_tokens))) return rc;
+  if ((rc = run_device_tokens(m, m->d_tokens, n_tokens, no_cache))) return rc;
   if (logits) {
     if (hipMemcpyAsync(logits, m->logits.p, (size_t)m->vocab * sizeof(float), hipMemcpyDeviceToHost, m->stream) !=
             hipSuccess ||

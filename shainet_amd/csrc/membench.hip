@@ -5,6 +5,10 @@
 // fp32 MFMAs does the same for the matrix cores: the rate they sustain at the clock
 // the device holds under that load, which the prefill kernels are compared with.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <algorithm>
+#include <vector>
 
 #include "../../include/shainet_hip_attn.h"
 
@@ -62,6 +66,11 @@ __global__ __launch_bounds__(512, 1) void mfma_f32_loop_kernel(float *__restrict
   sink[(long long)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// One workgroup of `lanes` lanes that does nothing: what a launch costs with no work in it.
+__global__ void empty_kernel(int *never) {
+  if (never && threadIdx.x == 12345) *never = 1;
+}
+
 }  // namespace
 
 extern "C" {
@@ -87,6 +96,34 @@ int shainet_hip_mfma_f32_loop(float *sink, int iters, int workgroups, long long 
   // 16 MFMAs per round and wavefront, 2 * 32 * 32 * 2 flops each, 8 wavefronts per workgroup
   if (flops) *flops = (long long)workgroups * 8 * iters * 16 * 4096;
   return hipGetLastError() == hipSuccess ? SHAINET_HIP_OK : SHAINET_HIP_ERR_RUNTIME;
+}
+
+int shainet_hip_launch_latency(int chain, int reps, int workgroups, float *us_out, void *stream_) {
+  if (chain < 1 || chain > 64 || reps < 1 || reps > 10000 || workgroups < 1 || !us_out) return SHAINET_HIP_ERR_ARGUMENT;
+  hipStream_t stream = (hipStream_t)stream_;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return SHAINET_HIP_ERR_RUNTIME;
+  std::vector<float> us;
+  int rc = SHAINET_HIP_OK;
+  for (int r = 0; r < reps + 3 && rc == SHAINET_HIP_OK; ++r) {
+    // the first kernel hands its own first clock reading to e0, the last its last one to e1
+    for (int i = 0; i < chain; ++i)
+      hipExtLaunchKernelGGL(empty_kernel, dim3((unsigned)workgroups), dim3(256), 0, stream, i == 0 ? e0 : nullptr,
+                            i == chain - 1 ? e1 : nullptr, 0, (int *)nullptr);
+    float ms = 0.f;
+    if (hipGetLastError() != hipSuccess || hipStreamSynchronize(stream) != hipSuccess ||
+        hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+      rc = SHAINET_HIP_ERR_RUNTIME;
+    else if (r >= 3)
+      us.push_back(ms * 1e3f);
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc == SHAINET_HIP_OK) {
+    std::sort(us.begin(), us.end());
+    *us_out = us[us.size() / 2];
+  }
+  return rc;
 }
 
 }  // extern "C"

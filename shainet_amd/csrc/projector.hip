@@ -1,6 +1,7 @@
 // Row-major projections on the device and small upload helpers.
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -191,7 +192,10 @@ int upload_side_by_side(float **dst, const float *const *mats, const int *widths
 // ---- the product by itself ---------------------------------------------------------------
 namespace {
 std::mutex g_matmul_lock;
-shainet::Projector g_matmul;  // grow-only scratch shared by the handle-less calls, like the reference's class-level scratch
+// Grow-only scratch of the handle-less calls (partial products of split shapes, their flag words, the
+// error word their kernels report into), one set per stream: calls on different streams may overlap
+// on the device and must not share partial products.  Never freed, like the reference's class-level scratch.
+std::map<hipStream_t, shainet::Projector> g_matmul;
 }  // namespace
 
 extern "C" int shainet_hip_matmul_f32(const float *x, long long x_stride, const float *w, const float *res, float *y,
@@ -201,11 +205,15 @@ extern "C" int shainet_hip_matmul_f32(const float *x, long long x_stride, const 
     return llama_fail(SHAINET_HIP_ERR_ARGUMENT, "invalid matmul arguments");
   if (!shainet_hip_available()) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
   std::lock_guard<std::mutex> guard(g_matmul_lock);
-  if (!g_matmul.error) g_matmul.error = alloc_error_word();
+  Projector &p = g_matmul[(hipStream_t)stream];
+  if (!p.error) p.error = alloc_error_word();
+  // what a kernel of an earlier call on this stream reported (a given-up wait for partial sums)
+  // is said by the next call, which does nothing else then
+  if (int rc = check_error_word(p.error)) return rc;
   Fused f;
   if (res) {
     f.epilogue = kGemvResidual;
     f.res = res;
   }
-  return g_matmul.project(x, x_stride, w, y, rows, k, n, (hipStream_t)stream, f);
+  return p.project(x, x_stride, w, y, rows, k, n, (hipStream_t)stream, f);
 }

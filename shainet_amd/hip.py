@@ -124,6 +124,7 @@ _SIGNATURES = {
     "shainet_llama_model_clear_cache": (C.c_int, [C.c_void_p]),
     "shainet_llama_model_cache_len": (C.c_int, [C.c_void_p]),
     "shainet_llama_model_run": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, _f32p]),
+    "shainet_llama_model_run_full": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.c_int, _f32p]),
     "shainet_llama_model_sync": (C.c_int, [C.c_void_p]),
     "shainet_llama_model_set_decode_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "shainet_llama_model_decode_mode_in_use": (C.c_int, [C.c_void_p]),
@@ -142,6 +143,7 @@ _SIGNATURES = {
     "shainet_hip_stream_copy_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_stream_read_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_void_p]),
     "shainet_hip_mfma_f32_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_longlong), C.c_void_p]),
+    "shainet_hip_launch_latency": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), C.c_void_p]),
     "shainet_attn_profile": (C.c_int, [C.c_void_p, C.c_int]),
     "shainet_attn_profile_read": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), _i32p]),
     "shainet_attn_profile_samples": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, _i32p]),
@@ -311,6 +313,14 @@ def mfma_f32_loop(sink, iters, workgroups=256, stream=None):
     flops = C.c_longlong(0)
     _check(lib().shainet_hip_mfma_f32_loop(_ptr(sink), iters, workgroups, C.byref(flops), stream))
     return flops.value
+
+
+def launch_latency(chain=1, reps=200, workgroups=256, stream=None):
+    """Microseconds from the first clock reading of the first of `chain` empty kernels to the last
+    reading of the last one (median of `reps` chains)."""
+    us = C.c_float(0)
+    _check(lib().shainet_hip_launch_latency(chain, reps, workgroups, C.byref(us), stream))
+    return us.value
 
 
 class AttnContext:
@@ -744,6 +754,17 @@ class LlamaModel:
         logits = np.empty(self.vocab, np.float32) if want_logits else None
         _check(lib().shainet_llama_model_run(self._h, ids.ctypes.data_as(C.POINTER(C.c_int)), ids.size,
                                              logits.ctypes.data_as(_f32p) if want_logits else None))
+        return logits
+
+    def run_full(self, tokens, want_logits=True):
+        """Network#run with use_kv_cache off: the rows attend among themselves from position 0,
+        the caches are not touched; returns the last row's logits like `run`."""
+        import numpy as np
+
+        ids = np.ascontiguousarray(tokens, np.int32).reshape(-1)
+        logits = np.empty(self.vocab, np.float32) if want_logits else None
+        _check(lib().shainet_llama_model_run_full(self._h, ids.ctypes.data_as(C.POINTER(C.c_int)), ids.size,
+                                                  logits.ctypes.data_as(_f32p) if want_logits else None))
         return logits
 
     def sync(self):

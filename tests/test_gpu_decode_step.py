@@ -218,8 +218,19 @@ def test_step_refuses_what_it_cannot_do(hip):
     with pytest.raises(hip.ArgumentError, match="lengths_to_device"):
         cache.lengths_from_device()
     cache.lengths_to_device()
+    # between the two copies the device's lengths are the ones that count: whatever reads or writes the
+    # host's copy is refused (it would drop or overwrite the rows the steps append)
+    for refused in (lambda: cache.reserve(128), lambda: cache.truncate(0, 5), lambda: cache.clear(),
+                    lambda: cache.fill(0, np.zeros((KV, 3, hd), np.float32), np.zeros((KV, 3, hd), np.float32)),
+                    lambda: ctx.forward(cache, q, k, v, [1]), lambda: cache.lengths_to_device()):
+        with pytest.raises(hip.ArgumentError, match="lengths_from_device"):
+            refused()
+    assert cache.len(0) == -1
+    ctx.decode_step(cache, q, k, v, torch.empty_like(q))
+    cache.lengths_from_device()
+    assert cache.len(0) == 11
     cache.reserve(128)
-    with pytest.raises(hip.ArgumentError, match="grown"):
+    with pytest.raises(hip.ArgumentError, match="lengths_to_device"):   # the lengths are back on the host
         ctx.decode_step(cache, q, k, v, torch.empty_like(q))
     q2, k2, v2 = _rows(torch, gen, 2, H, KV, hd)
     cache.lengths_to_device()

@@ -319,6 +319,42 @@ def test_tiny_llama_logits_match_transformers_and_oracle(hip, golden_dir):
         m.run([32000])
 
 
+def test_model_run_without_kv_cache_matches_fixture_and_oracle(hip, golden_dir):
+    """Network#run with use_kv_cache off at model level (network_run.cr:199-204, network_setup.cr:32):
+    every block takes LlamaBlock#forward, the caches stay as they are; and the reference's own
+    equivalence (spec/rope_kv_cache_spec.cr:29-59): cached prefill + decode gives the last row of
+    the full run."""
+    d = np.load(os.path.join(golden_dir, "tiny_llama_logits.npz"))
+    m, w = _tiny_model(hip)
+    om = tinyllama.OracleModel(w, orc)
+    t4 = [int(t) for t in d["tokens_t4"]]
+    full = m.run_full(t4)
+    assert m.cache_len == 0                                      # nothing was appended
+    assert np.abs(full - d["logits_t4"]).max() < 1e-5
+    rm.assert_close(full, om.run_full(t4), ATOL, RTOL, "no-cache logits")
+    np.testing.assert_array_equal(m.logits(), full)              # left for the sampler like run's
+    assert hip.Sampler.greedy(m) == orc.greedy(full)
+    # with rows in the caches: they neither take part nor change
+    m.run(t4[:3], want_logits=False)
+    om.run(t4[:3])
+    again = m.run_full(t4)
+    np.testing.assert_array_equal(again, full)
+    assert m.cache_len == 3
+    cached = m.run(t4[3:])                                       # decode on top of the cached prefill
+    rm.assert_close(cached, om.run(t4[3:]), ATOL, RTOL, "decode after a no-cache run")
+    assert np.abs(cached - full).max() < 2e-5                    # = the full run's last row
+    # a longer sequence (many rows take the MFMA product and the MFMA attention kernel), one row, errors
+    r = np.random.default_rng(4)
+    long = [int(t) for t in r.integers(0, 32000, 150)]
+    rm.assert_close(m.run_full(long), om.run_full(long), ATOL, RTOL, "150 rows without cache")
+    rm.assert_close(m.run_full(long[:1]), om.run_full(long[:1]), ATOL, RTOL, "one row without cache")
+    assert m.cache_len == 4
+    with pytest.raises(hip.ArgumentError):
+        m.run_full([32000])
+    with pytest.raises(hip.ArgumentError):
+        m.run_full([])
+
+
 def test_tiny_llama_greedy_generation_matches_oracle(hip):
     m, w = _tiny_model(hip)
     om = tinyllama.OracleModel(w, orc)

@@ -12,6 +12,8 @@ import prefill_cases as pc
 import refmath as rm
 from oracle import oracle as orc
 
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
 pytestmark = pytest.mark.gpu
 
 ATOL, RTOL = 1e-4, 1e-3
@@ -223,6 +225,26 @@ def test_decode_group_sizes(hip, g, hd):
     blocks[0].fill_cache(kf, vf)
     for _ in range(2):
         check_step(ctx, cache, blocks, r, [1])
+
+
+@pytest.mark.parametrize("H,KV,hd,norm", [(32, 1, 64, False), (64, 2, 128, True), (48, 2, 64, False)])
+def test_more_than_16_query_heads_per_kv_head(hip, H, KV, hd, norm):
+    """llama_block.cr:80 allows any divisor.  32 (or 24) query heads per kv head do not fit the 16
+    columns of the split-K decode kernel: such calls take the MFMA kernel (virtual rows = new rows x
+    heads of the group, key chunks + combine on a long cached prefix), also for one new row."""
+    ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=norm, capacity=1400, seed=H + hd)
+    kf, vf = (r.standard_normal((KV, 1100, hd)).astype(np.float32) for _ in range(2))
+    cache.fill(0, kf, vf)
+    blocks[0].fill_cache(kf, vf)
+    assert hip.describe_plan(H, KV, hd, [1100], [1])["path"] == hip.hip.PATH_PREFILL
+    for T in (1, 1, 40, 1, 3):
+        check_step(ctx, cache, blocks, r, [T], what=f"{H // KV} heads per kv head, {T} new rows")
+    check_cache_bits(cache, blocks)
+    # from an empty cache too
+    cache.clear()
+    blocks[0].clear_cache()
+    for T in (1, 17, 1):
+        check_step(ctx, cache, blocks, r, [T])
 
 
 @pytest.mark.parametrize("seed", range(10))
@@ -602,6 +624,35 @@ def test_reference_named_entry_points(hip, H, g, hd, S, T):
     torch.cuda.synchronize()
     rm.assert_close(out.cpu().numpy(), want, ATOL, RTOL)
     assert torch.equal(kc[:, S:S + T].cpu(), torch.from_numpy(k_new))
+
+
+def test_reference_named_attention_reports_a_given_up_wait(hip):
+    """attention_kv_f32 returns nothing and is asynchronous: what an earlier call's kernel reported is
+    printed by the next call, as the reference prints the launch error of every call
+    (cuda_kernels.cu:821-824).  Forced from the host in a child process (the switch is read when
+    the handle-less context is made): marks go where nobody looks, polling ends after 2000 looks."""
+    import subprocess
+    import sys
+
+    code = """
+import numpy as np, torch, shainet_amd as sa
+H, g, hd, S, cap = 8, 2, 64, 2500, 3000
+KV = H // g
+kc = torch.randn((KV, cap, hd), device="cuda"); vc = torch.randn((KV, cap, hd), device="cuda")
+q = torch.randn((1, H * hd), device="cuda"); out = torch.empty_like(q)
+torch.cuda.synchronize()
+for i in range(2):
+    sa.HIP.attention_kv_f32(q, kc, vc, out, None, 1, S, H, g, hd, cap, 0.125)
+    torch.cuda.synchronize()
+print("done")
+"""
+    env = dict(os.environ, SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS="1", PYTHONPATH=ROOT)
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and "done" in done.stdout, done.stderr[-2000:]
+    assert "HIP Error in attention_kv_f32 (an earlier call)" in done.stderr and "gave up waiting" in done.stderr, done.stderr[-2000:]
+    env.pop("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS")
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and "HIP Error" not in done.stderr, done.stderr[-2000:]
 
 
 def test_device_pointer_mode_matches_host_pointer_mode(hip):

@@ -90,6 +90,29 @@ def test_noalloc_matches_forward_two_calls_second_smaller(hip):
     assert np.all(np.abs(g - want) <= 1e-4 + 1e-3 * np.abs(want)), np.abs(g - want).max()
 
 
+def test_noalloc_allocates_no_device_memory(hip):
+    """Free device memory as the runtime reports it is the same before and after a run of calls
+    (contexts, caches and inputs are made first; shainet_attn_forward on a twin context, which
+    allocates its scratch on demand, shows that the probe sees such allocations)."""
+    import torch
+
+    H, KV, hd = 32, 8, 128
+    (ref, alt), gen = _pair(hip, H, KV, hd, [2900] * 8, 3000, seed=4)
+    rows = [_rows(torch, gen, 8, H, KV, hd) for _ in range(6)]
+    outs = [torch.empty_like(rows[0][0]) for _ in range(6)]
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for (q, k, v), out in zip(rows, outs):
+        alt[0].forward_noalloc(alt[1], q, k, v, [1] * 8, out=out)
+    alt[0].sync()
+    assert torch.cuda.mem_get_info()[0] == free0
+    wants = [ref[0].forward(ref[1], q, k, v, [1] * 8) for q, k, v in rows]
+    ref[0].sync()
+    assert torch.cuda.mem_get_info()[0] < free0       # rotated queries, partials, flags: grown on demand
+    for want, out in zip(wants, outs):
+        assert torch.equal(want, out)
+
+
 def _norms(seed, hd):
     r = np.random.default_rng(seed)
     return tuple((1 + 0.02 * r.standard_normal(hd)).astype(np.float32) for _ in range(2))

@@ -47,11 +47,16 @@ class OracleModel:
         for b in self.blocks:
             b.clear_cache()
 
-    def hidden(self, tokens):
+    def hidden(self, tokens, cached=True):
         x = self.orc.embed(self.w["embed"], tokens)
         for b, lw in zip(self.blocks, self.w["layers"]):
-            x = b.forward(x, lw["norm1"], lw["norm2"], self.eps, lw["gate"], lw["up"], lw["down"], True)
+            x = b.forward(x, lw["norm1"], lw["norm2"], self.eps, lw["gate"], lw["up"], lw["down"], cached)
         return x
 
     def run(self, tokens):
         return self.orc.logits_last(self.hidden(tokens), self.w["final_norm"], self.eps, self.w["lm_head"])
+
+    def run_full(self, tokens):
+        """Network#run with use_kv_cache off: LlamaBlock#forward in every block, caches untouched."""
+        return self.orc.logits_last(self.hidden(tokens, cached=False), self.w["final_norm"], self.eps,
+                                    self.w["lm_head"])
