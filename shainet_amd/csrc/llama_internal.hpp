@@ -88,6 +88,7 @@ struct Projector {
   void release();
 
  private:
+  int reserve_flags(size_t n_flags, hipStream_t stream);
   // res != nullptr: y = res + x W
   int gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N, hipStream_t stream,
            const float *res = nullptr);

@@ -63,12 +63,32 @@ void DevF::release() {
   cap = 0;
 }
 
+// The flag words are shared by all kernels of this projector: each leaves them zero, and the
+// launches of one projector follow each other on one stream.
+int Projector::reserve_flags(size_t n_flags, hipStream_t stream) {
+  if (n_flags <= flags_cap) return SHAINET_HIP_OK;
+  size_t want = flags_cap ? flags_cap : 4096;
+  while (want < n_flags) want *= 2;
+  unsigned *np = nullptr;
+  if (hipMalloc((void **)&np, want * sizeof(unsigned)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (hipMemsetAsync(np, 0, want * sizeof(unsigned), stream) != hipSuccess) {
+    (void)hipFree(np);
+    return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipMemsetAsync(flags) failed");
+  }
+  if (flags) (void)hipFree(flags);  // hipFree waits for the device
+  flags = np;
+  flags_cap = want;
+  return SHAINET_HIP_OK;
+}
+
 // y = (res +) x W with the library's own MFMA kernel; res == y is allowed.
 int Projector::gemm(const float *x, long long x_stride, const float *w, float *y, int T, int K, int N,
                     hipStream_t stream, const float *res) {
   const GemmPlan p = plan_gemm(T, K, N, x_stride);
   if (!scratch.reserve(p.partial_floats)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-  hipError_t e = launch_gemm(x, x_stride, w, y, res, scratch.p, T, K, N, p, stream);
+  if (int rc = reserve_flags(p.flag_words, stream)) return rc;
+  if (p.flag_words && !error) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "the projector has no error word");
+  hipError_t e = launch_gemm(x, x_stride, w, y, res, scratch.p, flags, error, T, K, N, p, stream);
   if (e != hipSuccess) return llama_fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemm launch: ") + hipGetErrorString(e));
   return SHAINET_HIP_OK;
 }
@@ -92,20 +112,8 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     }
     const GemvPlan p = plan_gemv(T, K, N, f.epilogue, f.prep ? f.prep->hd : 0);
     if (!scratch.reserve(p.partial_floats)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-    const size_t n_flags = (size_t)p.col_tiles * p.splits;
-    if (p.splits > 1 && n_flags > flags_cap) {
-      size_t want = flags_cap ? flags_cap : 4096;
-      while (want < n_flags) want *= 2;
-      unsigned *np = nullptr;
-      if (hipMalloc((void **)&np, want * sizeof(unsigned)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-      if (hipMemsetAsync(np, 0, want * sizeof(unsigned), stream) != hipSuccess) {
-        (void)hipFree(np);
-        return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipMemsetAsync(flags) failed");
-      }
-      if (flags) (void)hipFree(flags);  // hipFree waits for the device
-      flags = np;
-      flags_cap = want;
-    }
+    if (p.splits > 1)
+      if (int rc = reserve_flags((size_t)p.col_tiles * p.splits, stream)) return rc;
     if (p.splits > 1 && !error) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "the projector has no error word");
     GemvArgs a = {};
     a.x = xin;

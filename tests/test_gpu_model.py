@@ -161,11 +161,13 @@ def test_block_many_rows_take_the_mfma_product(hip):
     (40, 128, 128, True, None),
     (129, 64, 132, False, None),     # two row tiles, columns past a tile edge
     (300, 344, 128, True, None),     # K not a multiple of 32: the guarded loads
-    (255, 2048, 3072, False, None),  # the q | k | v product of the 1B shape: K cut into chunks
+    (255, 2048, 3072, False, None),  # the q | k | v product of the 1B shape: ten pieces per tile and the kernel that adds them
+    (700, 512, 640, True, None),     # 30 tiles of 16 steps: two workgroups per tile, the second adds the first's piece
+    (390, 1000, 1028, True, None),   # 36 tiles of 32 steps (the last one guarded), runs of units that cross tile ends
     (100, 30, 50, False, None),      # nothing a multiple of 4: the plain kernel
     (33, 128, 96, False, 160),       # rows of x at a stride
     (5, 256, 64, True, None),        # few rows: the split GEMV behind the same entry point
-    (24, 8192, 2048, True, None),    # the down projection of the 1B shape, 16 chunks along K
+    (24, 8192, 2048, True, None),    # the down projection of the 1B shape, 32 pieces along K
 ])
 def test_matmul_matches_oracle(hip, T, K, N, res, stride):
     """The projection product by itself against SimpleMatrix#* as the oracle restates it (fp64
@@ -199,14 +201,16 @@ def test_matmul_full_tiles_llama1b_prefill_shapes(hip):
     from shainet_amd import hip as binding
 
     g = torch.Generator(device="cuda").manual_seed(3)
-    for K, N in ((2048, 3072), (2048, 2048), (2048, 16384), (8192, 2048)):
-        x = torch.randn((512, K), generator=g, device="cuda")
+    # and 2048 rows of the first: 384 tiles, three quarters of what the chip runs at once, dealt out as equal runs of K steps
+    for T, K, N in ((512, 2048, 3072), (512, 2048, 2048), (512, 2048, 16384), (512, 8192, 2048), (2048, 2048, 3072)):
+        x = torch.randn((T, K), generator=g, device="cuda")
         w = torch.randn((K, N), generator=g, device="cuda") / K ** 0.5
         got = binding.matmul(x, w)
         want = (x.double() @ w.double()).float()
         torch.cuda.synchronize()
         err = (got - want).abs()
-        assert bool((err <= ATOL + RTOL * want.abs()).all()), f"K={K} N={N}: max err {err.max().item():.2e}"
+        assert bool((err <= ATOL + RTOL * want.abs()).all()), f"T={T} K={K} N={N}: max err {err.max().item():.2e}"
+        assert torch.equal(got, binding.matmul(x, w)), f"T={T} K={K} N={N}: two calls, different bits"
 
 
 def test_block_llama1b_shape_prefill_and_decode(hip):
