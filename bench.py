@@ -49,11 +49,14 @@ DECODE_WORKLOADS = [
     # not a BASELINE configuration: four new rows per sequence on the headline's caches (they go
     # through the split-K decode kernel as further columns of its tiles: the same bytes, HBM bound)
     ("qwen3_8b_decode_b16_4rows_ctx2048-8192", 32, 8, 128, 1e6, True, None, 4),
-    # not BASELINE configurations: head dims without an MFMA instantiation (one wavefront per row and
-    # head, llama_block.cr:80-89 accepts any head_dim) and 32 query heads per kv head (more columns
-    # than the decode kernel's tile: the MFMA prefill kernel serves it), to put a number on both
-    ("generic_hd96_decode_b1_ctx4096", 32, 8, 96, 5e5, False, [4096], 1),
-    ("generic_hd256_decode_b1_ctx4096", 16, 4, 256, 5e5, False, [4096], 1),
+    # not BASELINE configurations: head dims between the decode kernel's tile layouts (64, 128 and
+    # 256 wide; llama_block.cr:80-89 accepts any head_dim), which run in tiles padded to the next
+    # layout, alone and as a batch (Phi-3-mini's heads: 32 of 96, no grouping), and 32 query heads
+    # per kv head (more columns than the decode kernel's tile: the MFMA prefill kernel serves it)
+    ("hd96_decode_b1_ctx4096", 32, 8, 96, 5e5, False, [4096], 1),
+    ("hd256_decode_b1_ctx4096", 16, 4, 256, 5e5, False, [4096], 1),
+    ("phi3_hd96_decode_b16_ctx4096", 32, 32, 96, 1e4, False, [4096] * 16, 1),
+    ("gemma_hd256_decode_b16_ctx4096", 16, 8, 256, 1e4, False, [4096] * 16, 1),
     ("mqa_g32_hd128_decode_b1_ctx4096", 32, 1, 128, 5e5, False, [4096], 1),
 ]
 # name, H, KV, head_dim, rope theta, QK-norm, cached length per sequence, new rows per sequence

@@ -160,7 +160,7 @@ int shainet_attn_forward(shainet_attn_ctx *ctx, shainet_kv_cache *cache, const i
  * <= 524288 floats), 6 MiB for the split's partial results and 32 KiB of flag words (with the
  * default 256 workgroups: any batch of up to 64 sequences of head_dim <= 128).  Limits, each
  * refused with SHAINET_HIP_ERR_ARGUMENT or SHAINET_HIP_ERR_CAPACITY and a message, nothing
- * appended: head_dim 64 or 128; at most 32 / (num_heads / num_kv_heads) new rows per sequence
+ * appended: head_dim a multiple of 4 up to 256; at most 32 / (num_heads / num_kv_heads) new rows per sequence
  * (the calls the split-K decode kernel takes); every position below the max_positions the
  * context was created with; sizes within the array.  All calls on one GPU share the array:
  * two calls of this entry point that overlap in time on one GPU (different contexts on
@@ -188,7 +188,7 @@ int shainet_attn_forward_noalloc(shainet_attn_ctx *ctx, shainet_kv_cache *cache,
  *   Call it after anything that changes the lengths on the host (shainet_attn_forward, fill,
  *   clear, truncate) or the capacity (reserve), before the next step; not while capturing.
  * shainet_attn_decode_step: q [n_seqs, num_heads*head_dim], k, v [n_seqs, num_kv_heads*head_dim],
- *   out like q; device pointers, asynchronous on the context's stream.  head_dim 64 or 128.
+ *   out like q; device pointers, asynchronous on the context's stream.  head_dim a multiple of 4 up to 128.
  *   A step that finds a sequence at the cache's capacity appends nothing, writes no output and
  *   leaves the lengths alone, and so do the steps after it; shainet_kv_cache_lengths_from_device
  *   (or shainet_attn_sync) then returns SHAINET_HIP_ERR_CAPACITY.

@@ -603,12 +603,13 @@ bool decode_entries(const SeqTable &st, const Shape &sh, SeqTable &out) {
 }
 
 Path choose_path(const SeqTable &st, const Shape &sh) {
-  if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
   // a few new rows per sequence: rows x heads of a group fit the 16 columns of the split-K
   // kernel's MFMA tiles, which then streams K and V once for all of them; up to twice as many
-  // rows go to it as two entries (decode_entries), which still beats the key-chunked prefill
+  // rows go to it as two entries (decode_entries), which still beats the key-chunked prefill.
+  // Its tiles take any head dimension up to 256 that is a multiple of 4 (padded to 64, 128 or 256).
   SeqTable tmp;
-  if (decode_entries(st, sh, tmp)) return Path::kDecodeSplitK;
+  if (decode_tile_head_dim(sh.hd) && decode_entries(st, sh, tmp)) return Path::kDecodeSplitK;
+  if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
   return Path::kPrefillMfma;
 }
 

@@ -105,6 +105,10 @@ inline int device_plan_slots(int n_seqs, int KV) { return kDevicePlanWorkgroups 
 hipError_t launch_decode_plan(int *lens, int n_seqs, const Shape &sh, int rope_positions, DecodeDevicePlan *out,
                               int *error, hipStream_t stream);
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p);
+// The head dimension the split-K decode kernel lays its tiles out for when the data's is hd: 64,
+// 128 or 256, the first that holds hd (a multiple of 4; the rest of a tile is padding that costs
+// no memory traffic); 0 when none does.
+int decode_tile_head_dim(int hd);
 size_t decode_flag_words(const DecodePlan &p);
 
 // q_rot: rotated queries [rows][H*hd]; the cache already holds the new rows.

@@ -305,7 +305,7 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
   if (ws && path != Path::kDecodeSplitK)
     return fail(SHAINET_HIP_ERR_ARGUMENT,
                 "the entry point that allocates nothing takes decode calls only: at most %d new rows per sequence "
-                "with this head geometry (head_dim 64 or 128)", 32 / (sh.g < 1 ? 1 : sh.g));
+                "with this head geometry (head_dim a multiple of 4 up to 256)", 32 / (sh.g < 1 ? 1 : sh.g));
   // the MFMA prefill kernels address the rows of a (sequence, kv head) by a 32-bit byte offset;
   // said before anything is written to the cache
   if (path == Path::kPrefillMfma && (long long)sh.cap * sh.hd * 4 > 0xffffffffLL)
@@ -928,8 +928,9 @@ DecodePlan step_launch_plan(const shainet_attn_ctx *c, int n_seqs) {
 extern "C" int shainet_kv_cache_lengths_to_device(shainet_kv_cache *kc) {
   if (!kc) return fail(SHAINET_HIP_ERR_ARGUMENT, "cache is null");
   shainet_attn_ctx *c = kc->ctx;
-  if ((c->hd != 64 && c->hd != 128) || c->g > 16)
-    return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps need head_dim 64 or 128 and at most 16 query heads per kv head");
+  if (!decode_tile_head_dim(c->hd) || c->hd > 128 || c->g > 16)  // (the step's prep kernel: a wavefront per row of at most 128)
+    return fail(SHAINET_HIP_ERR_ARGUMENT,
+                "decode steps need a head_dim that is a multiple of 4 up to 128 and at most 16 query heads per kv head");
   if (kc->batch > SHAINET_HIP_MAX_BATCH)
     return fail(SHAINET_HIP_ERR_ARGUMENT, "decode steps take caches of at most %d sequences", SHAINET_HIP_MAX_BATCH);
   StepState &st = kc->step;

@@ -86,28 +86,39 @@ struct DecodeCfg {
 // 181 -> 162 us with every sequence at 8192; the cache-scope bits on top of it change nothing.
 constexpr int kNonTemporal = 2;  // the nt bit of the cache-policy operand
 
+// PAD: the head dimension hd of the data is any multiple of 4 up to HD, the head dimension the
+// tiles are laid out for.  The query's elements beyond hd are zeros, so whatever stands in for
+// the keys' there does not reach the scores, and output elements beyond hd are never stored;
+// the pieces of a tile beyond hd repeat the row's first piece (a cache hit, no HBM traffic).
+// Without PAD hd == HD and no instruction is spent on any of this.
+//
 // Issue the asynchronous copy of the K tile starting at row `kb` into `lds`.
-template <int HD>
-__device__ __forceinline__ void issue_k_tile(const float *kbase, int kb, int last_row, char *lds, int lane) {
+template <int HD, bool PAD>
+__device__ __forceinline__ void issue_k_tile(const float *kbase, int kb, int last_row, char *lds, int lane, int hd) {
   using C = DecodeCfg<HD>;
 #pragma unroll
   for (int u = 0; u < C::NKI; ++u) {
     const int slot = u * 64 + lane;
     const int row = slot / C::PPR, q = slot % C::PPR;
-    const int piece = q ^ row;  // row < 16 only touches the low four bits
-    const float *src = kbase + (long long)min(kb + row, last_row) * HD + 4 * piece;
+    int piece = q ^ row;  // row < 16 only touches the low four bits
+    if (PAD) piece = 4 * piece < hd ? piece : 0;
+    const float *src = kbase + (long long)min(kb + row, last_row) * (PAD ? hd : HD) + 4 * piece;
     __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src), LDS_PTR(lds + u * 1024), 16, 0, kNonTemporal);
   }
 }
 
-template <int HD>
+template <int HD, bool PAD>
 __device__ __forceinline__ void load_v_tile(const float *vbase, int kb, int last_row, int col, int j,
-                                            f32x4 (&v)[4][DecodeCfg<HD>::NVU]) {
+                                            f32x4 (&v)[4][DecodeCfg<HD>::NVU], int hd) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const float *vp = vbase + (long long)min(kb + 4 * j + r, last_row) * HD + 4 * col;
+    const float *vp = vbase + (long long)min(kb + 4 * j + r, last_row) * (PAD ? hd : HD);
 #pragma unroll
-    for (int u = 0; u < DecodeCfg<HD>::NVU; ++u) v[r][u] = __builtin_nontemporal_load((const f32x4 *)(vp + 64 * u));
+    for (int u = 0; u < DecodeCfg<HD>::NVU; ++u) {
+      int d = 4 * col + 64 * u;
+      if (PAD) d = d < hd ? d : 0;
+      v[r][u] = __builtin_nontemporal_load((const f32x4 *)(vp + d));
+    }
   }
 }
 
@@ -174,8 +185,8 @@ constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each: s
 // same as part_flag except in the test of that give-up, which sends them elsewhere.
 // DEV: the sequence table and the spans come from *dev (device memory, written by
 // decode_plan_kernel earlier on the stream) instead of from the kernel arguments.
-template <int HD, int NW, bool DEV>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel(
+template <int HD, int NW, bool DEV, bool PAD>
+__global__ __launch_bounds__(64 * NW, NW == 4 && HD <= 128 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
     int spin_limit, int *error, SeqTable st_arg, Shape sh, int tiles_per_wg_arg, SpanTable sp_arg, int total_tiles_arg,
@@ -198,6 +209,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: tile numbers stay in scalar registers
   const int col = lane & 15, j = lane >> 4;
   const int g = sh.g;
+  const int hd = PAD ? sh.hd : HD;  // floats between two rows of q, K, V and the output
   const int t_begin = span_begin(blockIdx.x, tiles_per_wg, sp);
   const int t_end = min(total_tiles, span_begin(blockIdx.x + 1, tiles_per_wg, sp));
   if (t_begin >= t_end) return;  // unequal spans can leave the last workgroup without tiles
@@ -208,7 +220,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   // along them with dependent scalar loads took 2.5 us for a workgroup in the middle of 16
   // sequences).
   int s = (int)__popcll(__ballot(lane + 1 < st.n_seqs && t_begin >= st.work_off[lane + 1 < kMaxSeqs ? lane + 1 : kMaxSeqs]));
-  Segment seg = segment_at(t, t_end, s, st, sh, HD, kc, vc, rotate);
+  Segment seg = segment_at(t, t_end, s, st, sh, hd, kc, vc, rotate);
 
   f32x4 v_next[4][C::NVU];
   float qr[HD / 4];
@@ -217,10 +229,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   // MFMA column c of a segment is new row c / g, head c % g of the group (R * g <= 16 columns)
   auto load_q = [&](const Segment &sg) {
     const int cq = col < sg.R * g ? col : 0, row = cq / g;
-    const float *qp = q_rot + ((long long)(sg.token + row) * sh.H + sg.kvh * g + (cq - row * g)) * HD + 4 * j;
+    const float *qp = q_rot + ((long long)(sg.token + row) * sh.H + sg.kvh * g + (cq - row * g)) * hd + 4 * j;
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      const f32x4 x = *(const f32x4 *)(qp + 16 * i);
+      f32x4 x = {0.f, 0.f, 0.f, 0.f};
+      if (!PAD || 16 * i + 4 * j < hd) x = *(const f32x4 *)(qp + 16 * i);
       qr[4 * i + 0] = x.x;
       qr[4 * i + 1] = x.y;
       qr[4 * i + 2] = x.z;
@@ -242,8 +255,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
   static_assert((NW & (NW - 1)) == 0, "round-robin by masking");
   // start fetching the tile at key row `row` into buffer `which`
   auto fetch = [&](int which, const float *kb_, const float *vb_, int row, int last_row) {
-    issue_k_tile<HD>(kb_, row, last_row, my_lds + which * C::TILE_BYTES, lane);
-    load_v_tile<HD>(vb_, row, last_row, col, j, v_next);
+    issue_k_tile<HD, PAD>(kb_, row, last_row, my_lds + which * C::TILE_BYTES, lane, hd);
+    load_v_tile<HD, PAD>(vb_, row, last_row, col, j, v_next, hd);
   };
   if (first_place(t) < seg.tile1 - seg.tile0) fetch(0, seg.kbase, seg.vbase, tile_at(seg, first_place(t)) * 16, seg.L - 1);
   load_q(seg);
@@ -272,7 +285,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
     const int t_next = t + (tile1 - seg.tile0);
     const bool more = t_next < t_end;
     Segment nseg = seg;
-    if (more) nseg = segment_at(t_next, t_end, s, st, sh, HD, kc, vc, rotate);
+    if (more) nseg = segment_at(t_next, t_end, s, st, sh, hd, kc, vc, rotate);
     const int nplace = first_place(t_next);
     const bool nhave = more && nplace < nseg.tile1 - nseg.tile0;
     const int ntile = nhave ? tile_at(nseg, nplace) : 0;
@@ -390,7 +403,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
       }
       if (whole_pair) {
         const int row = cc / g;
-        out[((long long)(seg.token + row) * sh.H + seg.kvh * g + (cc - row * g)) * HD + d] = acc / ls;
+        if (!PAD || d < hd) out[((long long)(seg.token + row) * sh.H + seg.kvh * g + (cc - row * g)) * hd + d] = acc / ls;
       } else if (slot < n_slots) {
         const long long pi = (long long)slot * pstride + cc;
         coherent_store(&part_o[pi * HD + d], acc);
@@ -501,10 +514,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void decode_splitk_kernel
         acc.w += __shfl_xor(acc.w, o2);
         ls += __shfl_xor(ls, o2);
       }
-      if (grp == 0) {
+      if (grp == 0 && (!PAD || 4 * d4 < hd)) {
         const float inv = 1.0f / ls;
         const int row = cc / g;
-        *(f32x4 *)&out[((long long)(mseg.token + row) * sh.H + mseg.kvh * g + (cc - row * g)) * HD + 4 * d4] = acc * inv;
+        *(f32x4 *)&out[((long long)(mseg.token + row) * sh.H + mseg.kvh * g + (cc - row * g)) * hd + 4 * d4] = acc * inv;
       }
     }
   }
@@ -634,8 +647,14 @@ DecodePlan plan_decode(SeqTable &st, const Shape &sh, int wg_target) {
 
 size_t decode_flag_words(const DecodePlan &p) { return (size_t)p.n_slots * kDecodeWaves; }
 
+// The head dimension the split-K kernel's tiles are laid out for: 64, 128 or 256 (0: none fits).
+int decode_tile_head_dim(int hd) {
+  if (hd < 4 || (hd & 3) || hd > 256) return 0;
+  return hd <= 64 ? 64 : hd <= 128 ? 128 : 256;
+}
+
 size_t decode_partial_floats(const Shape &sh, const DecodePlan &p) {
-  return (size_t)p.n_slots * p.cols * (sh.hd + 2);
+  return (size_t)p.n_slots * p.cols * (decode_tile_head_dim(sh.hd) + 2);
 }
 
 hipError_t launch_decode_plan(int *lens, int n_seqs, const Shape &sh, int rope_positions, DecodeDevicePlan *out,
@@ -651,7 +670,7 @@ hipError_t launch_decode_plan(int *lens, int n_seqs, const Shape &sh, int rope_p
 hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &sh, const DecodePlan &p, float scale,
                          hipStream_t stream, hipEvent_t before, hipEvent_t after, const DecodeDevicePlan *dev) {
   if (st.n_seqs < 1 || st.n_seqs > kMaxSeqs || sh.g < 1 || sh.g > 16 || sh.H != sh.KV * sh.g ||
-      (sh.hd != 64 && sh.hd != 128) || p.n_wgs < 1 || !d.partials || !d.part_flag || !d.error)
+      !decode_tile_head_dim(sh.hd) || p.n_wgs < 1 || !d.partials || !d.part_flag || !d.error)
     return hipErrorInvalidValue;
   if (dev) {
     if (p.n_wgs != kDevicePlanWorkgroups || p.n_slots != device_plan_slots(st.n_seqs, sh.KV) || p.cols < sh.g)
@@ -667,7 +686,8 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   unsigned *flag_set = d.flag_set ? d.flag_set : d.part_flag;
   const int spin_limit = d.spin_limit > 0 ? d.spin_limit : kFlagSpinLimit;
   float *part_o = d.partials;
-  float *part_ml = d.partials + (size_t)p.n_slots * p.cols * sh.hd;
+  const int tile_hd = decode_tile_head_dim(sh.hd);
+  float *part_ml = d.partials + (size_t)p.n_slots * p.cols * tile_hd;
   const float c = scale * kLog2e;
   // before / after (nullable) receive the kernel's own first and last clock reading, not the
   // time at which the stream reached them: what is between two kernels stays out
@@ -678,21 +698,28 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
                                  : getenv("SHAINET_HIP_DECODE_ROTATE")
                                      ? (unsigned)atoi(getenv("SHAINET_HIP_DECODE_ROTATE"))
                                      : 0x7fffffffu;
-#define SHAINET_DECODE_LAUNCH(HD_, DEV_)                                                                            \
-  SHAINET_LAUNCH_TIMED((decode_splitk_kernel<HD_, kDecodeWaves, DEV_>), grid, block, 0, stream, before, after,     \
-                       d.q_rot, d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, \
-                       sh, p.tiles_per_wg, p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev)
-  if (sh.hd == 64) {
-    if (dev)
-      SHAINET_DECODE_LAUNCH(64, true);
-    else
-      SHAINET_DECODE_LAUNCH(64, false);
-  } else {
-    if (dev)
-      SHAINET_DECODE_LAUNCH(128, true);
-    else
-      SHAINET_DECODE_LAUNCH(128, false);
-  }
+#define SHAINET_DECODE_LAUNCH(HD_, DEV_, PAD_)                                                                      \
+  SHAINET_LAUNCH_TIMED((decode_splitk_kernel<HD_, kDecodeWaves, DEV_, PAD_>), grid, block, 0, stream, before,      \
+                       after, d.q_rot, d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit,       \
+                       d.error, st, sh, p.tiles_per_wg, p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev)
+#define SHAINET_DECODE_LAUNCH_HD(HD_, PAD_) \
+  do {                                      \
+    if (dev)                                \
+      SHAINET_DECODE_LAUNCH(HD_, true, PAD_);  \
+    else                                    \
+      SHAINET_DECODE_LAUNCH(HD_, false, PAD_); \
+  } while (0)
+  if (sh.hd == 64)
+    SHAINET_DECODE_LAUNCH_HD(64, false);
+  else if (sh.hd == 128)
+    SHAINET_DECODE_LAUNCH_HD(128, false);
+  else if (tile_hd == 64)
+    SHAINET_DECODE_LAUNCH_HD(64, true);
+  else if (tile_hd == 128)
+    SHAINET_DECODE_LAUNCH_HD(128, true);
+  else
+    SHAINET_DECODE_LAUNCH_HD(256, true);
+#undef SHAINET_DECODE_LAUNCH_HD
 #undef SHAINET_DECODE_LAUNCH
   return hipGetLastError();
 }

@@ -71,6 +71,9 @@ CASES = [
     (14, 2, 64, [700, 5, 90], False, True),                   # Qwen2.5-0.5B heads: g = 7, biases
     (8, 8, 128, [int(x) for x in np.random.default_rng(3).integers(1, 1500, 64)], False, False),  # 64 sequences, g = 1
     (32, 2, 128, [513, 64], True, False),                     # g = 16
+    (32, 8, 96, [700, 33, 1], True, True),                    # head_dim 96: tiles padded to 128
+    (8, 4, 44, [300, 2000], False, False),                    # head_dim 44: tiles padded to 64
+    (8, 2, 8, [40], False, False),                            # head_dim 8: tiles padded to 64
 ]
 
 
@@ -236,6 +239,7 @@ def test_step_refuses_what_it_cannot_do(hip):
     cache.lengths_to_device()
     with pytest.raises(hip.ArgumentError, match="n_seqs"):
         ctx.decode_step(cache, q2, k2, v2, torch.empty_like(q2))
-    odd = hip.AttnContext(4, 4, 32, rope_theta=1e4, max_positions=64)
-    with pytest.raises(hip.ArgumentError, match="head_dim"):
-        hip.KVCache(odd, 1, 64).lengths_to_device()
+    for odd_hd in (6, 256):   # not a multiple of 4; above 128
+        odd = hip.AttnContext(4, 4, odd_hd, rope_theta=1e4, max_positions=64)
+        with pytest.raises(hip.ArgumentError, match="head_dim"):
+            hip.KVCache(odd, 1, 64).lengths_to_device()

@@ -216,7 +216,9 @@ def test_decode_every_length_around_tile_and_chunk_edges(hip):
         check_step(ctx, cache, blocks, r, [1], threads=1, what=f"len {i + 1}")
 
 
-@pytest.mark.parametrize("g,hd", [(1, 64), (2, 128), (8, 128), (16, 64)])
+@pytest.mark.parametrize("g,hd", [(1, 64), (2, 128), (8, 128), (16, 64),
+                                  # head dimensions between the tile layouts (64, 128, 256 wide): padded tiles
+                                  (4, 96), (2, 256), (8, 32), (1, 8), (3, 80), (4, 200), (2, 132)])
 def test_decode_group_sizes(hip, g, hd):
     KV = 2
     ctx, cache, blocks, r = make_pair(hip, KV * g, KV, hd, 1e6, capacity=1500, seed=g)
@@ -284,6 +286,9 @@ def test_decode_random_ragged_batches(hip, seed):
     (8, 4, 128, 16, [8, 5, 7, 1] * 4, 900),         # more rows than one tile has columns: two entries each
     (2, 8, 64, 3, [4, 3, 1], 600),
     (4, 1, 64, 2, [32, 17], 300),
+    (4, 4, 96, 6, [1, 4, 2, 8, 3, 1], 700),         # a head dimension the tiles are padded for (Phi-3-mini's)
+    (2, 2, 256, 3, [5, 1, 16], 500),                # Gemma's
+    (4, 2, 24, 2, [3, 1], 100),
 ])
 def test_few_new_rows_take_the_decode_split(hip, KV, g, hd, B, rows_new, top):
     """A few new rows per sequence (rows x heads of a group <= 16) go through the split-K decode

@@ -92,8 +92,8 @@ def test_noalloc_matches_forward_two_calls_second_smaller(hip):
 
 def test_noalloc_allocates_no_device_memory(hip):
     """Free device memory as the runtime reports it is the same before and after a run of calls
-    (contexts, caches and inputs are made first; shainet_attn_forward on a twin context, which
-    allocates its scratch on demand, shows that the probe sees such allocations)."""
+    (contexts, caches and inputs are made first; another cache made afterwards shows that the probe
+    sees what the library allocates)."""
     import torch
 
     H, KV, hd = 32, 8, 128
@@ -108,7 +108,9 @@ def test_noalloc_allocates_no_device_memory(hip):
     assert torch.cuda.mem_get_info()[0] == free0
     wants = [ref[0].forward(ref[1], q, k, v, [1] * 8) for q, k, v in rows]
     ref[0].sync()
-    assert torch.cuda.mem_get_info()[0] < free0       # rotated queries, partials, flags: grown on demand
+    extra = hip.KVCache(ref[0], 8, 3000)              # 196 MB from hipMalloc
+    assert torch.cuda.mem_get_info()[0] < free0
+    del extra
     for want, out in zip(wants, outs):
         assert torch.equal(want, out)
 
