@@ -66,6 +66,8 @@ PREFILL_WORKLOADS = [
     ("qwen3_30b_chunked_prefill_t512_on_16384", 32, 4, 128, 1e6, True, [16384], 512),
     # not a BASELINE configuration: the headline model's shape (QK-norm, head_dim 128) from an empty cache
     ("qwen3_8b_prefill_t2048", 32, 8, 128, 1e6, True, [0], 2048),
+    # not a BASELINE configuration: Phi-3-mini's heads (32 of head_dim 96, no grouping) in tiles padded to 128
+    ("phi3_hd96_prefill_t2048", 32, 32, 96, 1e4, False, [0], 2048),
 ]
 
 
@@ -563,7 +565,8 @@ def main():
             results[name] = w.run_decode(K if len(lens) < 16 else max(20, K // 2), W)
             w.close()
     fewer = {"llama1b_prefill_t2048": K, "llama1b_prefill_t8192": max(5, K // 20),
-             "qwen3_30b_chunked_prefill_t512_on_16384": max(5, K // 10), "qwen3_8b_prefill_t2048": max(5, K // 2)}
+             "qwen3_30b_chunked_prefill_t512_on_16384": max(5, K // 10), "qwen3_8b_prefill_t2048": max(5, K // 2),
+             "phi3_hd96_prefill_t2048": max(5, K // 4)}
     for name, H, KV, hd, th, norm, lens, T in PREFILL_WORKLOADS:
         if want(name):
             w = Workload(sa, torch, name, H, KV, hd, th, norm, lens3 if lens is None else lens, T, 7)

@@ -214,7 +214,8 @@ int shainet_attn_last_q_rot(shainet_attn_ctx *ctx, float *out, int rows);
 /* What a shainet_attn_forward call with these sequences (cached positions start_pos[s], new rows
  * new_tokens[s]) launches for its attention step, without launching anything; needs no device.
  * plan[0] path: 0 = split-K decode kernel, 1 = MFMA prefill kernel, 2 = generic kernel;
- * plan[1] head_dim; plan[2] key chunks per row block (1 = none, > 1 adds the combine kernel);
+ * plan[1] the head_dim the kernel's tiles are laid out for (64, 128 or 256: the first that holds
+ * head_dim; head_dim itself on the generic path); plan[2] key chunks per row block (1 = none, > 1 adds the combine kernel);
  * plan[3] wavefront groups per workgroup (1 = four wavefronts, 2 = eight); plan[4] row blocks a
  * workgroup takes in turn (0 = one workgroup per block and chunk); plan[5] workgroups;
  * plan[6] decode: 16-key tiles per workgroup, prefill: row blocks; plan[7] workgroups per

@@ -80,7 +80,11 @@ __device__ __forceinline__ void locate_block(const SeqTable &st, int rank, int &
 // do not hide: fp32 MFMAs and vector instructions share the SIMD's lanes).  The two
 // halves merge through LDS.
 // One workgroup's work: the row block (and key chunk) number `bid` of the launch.
-template <int HD, bool SPLIT, int G>
+// PAD: the head dimension of the data (sh.hd, a multiple of 4) is smaller than HD, the one the
+// tiles are laid out for: query elements beyond it are zeros (whatever stands in for the keys'
+// there does not reach the scores), output elements beyond it are not stored, and a tile's
+// pieces beyond it repeat the row's first piece (a cache hit, no HBM traffic).
+template <int HD, bool SPLIT, int G, bool PAD>
 __device__ __forceinline__ void prefill_block(const int bid, const float *__restrict__ q_rot,
                                               const float *__restrict__ kc, const float *__restrict__ vc,
                                               float *__restrict__ out, float *__restrict__ part_o,
@@ -131,10 +135,11 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   const int n_tiles = wg_hi / 32 + 1;
   const int tiles_per_chunk = SPLIT ? (n_tiles + ns - 1) / ns : n_tiles;
   const int kt0 = chunk * tiles_per_chunk, kt1 = min(n_tiles, kt0 + tiles_per_chunk);
-  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * HD;
+  const int hd = PAD ? uniform(sh.hd) : HD;  // floats between two rows of q, K, V and the output
+  const long long head_base = (long long)st.slot[s] * sh.seq_stride + (long long)kvh * sh.cap * hd;
   const float *kbase = kc + head_base;
   const float *vbase = vc + head_base;
-  const long long qo_off = ((long long)(st.tok_off[s] + row) * sh.H + kvh * g + hg) * HD;
+  const long long qo_off = ((long long)(st.tok_off[s] + row) * sh.H + kvh * g + hg) * hd;
 
   float qr[HD / 2];
   {
@@ -144,7 +149,8 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
       // (lanes past the last virtual row repeat the last row: their results are never used,
       // and not touching the loaded values here lets the first K and V loads go out behind
       // these instead of after their arrival)
-      const f32x4 t = *(const f32x4 *)(qp + 8 * i);
+      f32x4 t = {0.f, 0.f, 0.f, 0.f};
+      if (!PAD || 8 * i + 4 * j < hd) t = *(const f32x4 *)(qp + 8 * i);
       qr[4 * i + 0] = t.x;
       qr[4 * i + 1] = t.y;
       qr[4 * i + 2] = t.z;
@@ -192,7 +198,8 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     const int ts = idx / TILE4, rem = idx - ts * TILE4;
     row_in_step[u] = ts * 32 + rem / (HD / 4);
   }
-  const unsigned col_bytes = 16u * (threadIdx.x % (HD / 4));  // NTHREADS is a multiple of HD / 4
+  // NTHREADS is a multiple of HD / 4
+  const unsigned col_bytes = PAD && 4 * (threadIdx.x % (HD / 4)) >= (unsigned)hd ? 0u : 16u * (threadIdx.x % (HD / 4));
   static_assert(NTHREADS % (HD / 4) == 0, "a thread keeps its columns");
   // a scalar base and a 32-bit byte offset per lane (a head's rows span less than 4 GiB: checked
   // at launch); rows past the last one repeat it
@@ -200,7 +207,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
     const int first_row = (kt0 + G * sp) * 32;
 #pragma unroll
     for (int u = 0; u < LD4; ++u) {
-      const unsigned off = (unsigned)min(first_row + row_in_step[u], L - 1) * (unsigned)(HD * 4) + col_bytes;
+      const unsigned off = (unsigned)min(first_row + row_in_step[u], L - 1) * (unsigned)(hd * 4) + col_bytes;
       dst[u] = *(const f32x4 *)((const char *)base + off);
     }
   };
@@ -426,6 +433,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int d = NT * (8 * (r >> 2) + 4 * j + (r & 3));
+      if (PAD && d >= hd) continue;  // (hd is a multiple of 4 and d of NT = 2 or 4: a store lies inside or outside as a whole)
       if constexpr (NT == 2) {
         *(float2 *)(op + d) = float2{o[0][r] * inv, o[1][r] * inv};
       } else {
@@ -435,7 +443,7 @@ __device__ __forceinline__ void prefill_block(const int bid, const float *__rest
   }
 }
 
-template <int HD, bool SPLIT, int G>
+template <int HD, bool SPLIT, int G, bool PAD>
 __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(const float *__restrict__ q_rot,
                                                               const float *__restrict__ kc,
                                                               const float *__restrict__ vc,
@@ -443,7 +451,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
                                                               float *__restrict__ part_o,
                                                               float *__restrict__ part_ml, SeqTable st,
                                                               Shape sh, int ns, float c) {
-  prefill_block<HD, SPLIT, G>(blockIdx.x, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);
+  prefill_block<HD, SPLIT, G, PAD>(blockIdx.x, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);
 }
 
 // For launches of two or three row blocks per compute unit: a workgroup takes, in turn, block b
@@ -451,7 +459,7 @@ __global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void prefill_mfma_kernel(c
 // 2N + b (N workgroups): long, short and shorter ones that add up to about the same work for
 // every workgroup, instead of the dispatcher starting another workgroup where one has ended
 // (3.5 us later, measured).
-template <int HD, int G>
+template <int HD, int G, bool PAD>
 __global__ __launch_bounds__(256 * G, 1) void prefill_turns_kernel(const float *__restrict__ q_rot,
                                                                    const float *__restrict__ kc,
                                                                    const float *__restrict__ vc,
@@ -462,7 +470,7 @@ __global__ __launch_bounds__(256 * G, 1) void prefill_turns_kernel(const float *
     const int bid = (turn & 1) ? (turn + 1) * N - 1 - b : turn * N + b;
     if (bid >= n_blocks) continue;
     if (turn) __syncthreads();  // the LDS stages are free: nobody is still merging the last block's halves
-    prefill_block<HD, false, G>(bid, q_rot, kc, vc, out, nullptr, nullptr, st, sh, 1, c);
+    prefill_block<HD, false, G, PAD>(bid, q_rot, kc, vc, out, nullptr, nullptr, st, sh, 1, c);
   }
 }
 
@@ -472,7 +480,8 @@ __global__ __launch_bounds__(256 * G, 1) void prefill_turns_kernel(const float *
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ part_o,
                                                               const float *__restrict__ part_ml,
                                                               float *__restrict__ out, SeqTable st, Shape sh,
-                                                              int ns, float c) {
+                                                              int ns, float c, int tile_hd) {
+  // tile_hd: floats per row of a partial (the head dimension the tiles were laid out for)
   const int kvh = blockIdx.x % sh.KV, item = blockIdx.x / sh.KV;
   int s, vb;
   locate_block(st, item, s, vb);
@@ -500,7 +509,7 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__res
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const long long pi = base + (long long)min(k0 + u, ns - 1) * 128 + vl;
-        x[u] = *(const f32x4 *)(part_o + pi * hd + 4 * d4);
+        x[u] = *(const f32x4 *)(part_o + pi * tile_hd + 4 * d4);
         mk[u] = part_ml[2 * pi];
         lk[u] = part_ml[2 * pi + 1];
       }
@@ -602,6 +611,11 @@ bool decode_entries(const SeqTable &st, const Shape &sh, SeqTable &out) {
   return true;
 }
 
+int prefill_tile_head_dim(int hd) {
+  if (hd < 4 || (hd & 3) || hd > 128) return 0;
+  return hd <= 64 ? 64 : 128;
+}
+
 Path choose_path(const SeqTable &st, const Shape &sh) {
   // a few new rows per sequence: rows x heads of a group fit the 16 columns of the split-K
   // kernel's MFMA tiles, which then streams K and V once for all of them; up to twice as many
@@ -609,7 +623,8 @@ Path choose_path(const SeqTable &st, const Shape &sh) {
   // Its tiles take any head dimension up to 256 that is a multiple of 4 (padded to 64, 128 or 256).
   SeqTable tmp;
   if (decode_tile_head_dim(sh.hd) && decode_entries(st, sh, tmp)) return Path::kDecodeSplitK;
-  if (sh.hd != 64 && sh.hd != 128) return Path::kGeneric;
+  // the MFMA prefill kernel's tiles: head dimensions up to 128 (padded to 64 or 128)
+  if (!prefill_tile_head_dim(sh.hd)) return Path::kGeneric;
   return Path::kPrefillMfma;
 }
 
@@ -669,7 +684,7 @@ int prefill_key_splits(const SeqTable &st, const Shape &sh, int items) {
 }
 
 size_t prefill_partial_floats(const Shape &sh, int items, int ns) {
-  return ns > 1 ? (size_t)items * sh.KV * ns * 128 * (sh.hd + 2) : 0;
+  return ns > 1 ? (size_t)items * sh.KV * ns * 128 * (prefill_tile_head_dim(sh.hd) + 2) : 0;
 }
 
 PrefillLaunch plan_prefill_launch(const Shape &sh, int items, int ns, int wgs_per_cu, int groups) {
@@ -680,7 +695,8 @@ PrefillLaunch plan_prefill_launch(const Shape &sh, int items, int ns, int wgs_pe
   // two per SIMD (G = 2).  Larger launches already have several workgroups per unit.
   p.groups = groups == 1 || groups == 2 ? groups : (p.n_wgs <= 768 ? 2 : 1);
   // static LDS of the kernel: two stages of `groups` padded K tiles and V tiles
-  const size_t static_lds = (size_t)2 * p.groups * (32 * (sh.hd + 4) + 32 * sh.hd) * sizeof(float);
+  const int tile_hd = prefill_tile_head_dim(sh.hd);
+  const size_t static_lds = (size_t)2 * p.groups * (32 * (tile_hd + 4) + 32 * tile_hd) * sizeof(float);
   p.pad = 0;
   // With fewer workgroups than three per compute unit everything is resident at
   // once and the dispatcher cannot balance the triangular work: one workgroup per
@@ -706,8 +722,9 @@ PrefillLaunch plan_prefill_launch(const Shape &sh, int items, int ns, int wgs_pe
 hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, float *out, float *partials,
                           const SeqTable &st, const Shape &sh, int items, int ns, float scale,
                           hipStream_t stream, int wgs_per_cu, int groups_wanted, hipEvent_t before, hipEvent_t after) {
-  if (!table_ok(st, sh) || (sh.hd != 64 && sh.hd != 128) || items < 1 || ns < 1 || (ns > 1 && !partials))
-    return hipErrorInvalidValue;
+  const int tile_hd = prefill_tile_head_dim(sh.hd);
+  if (!table_ok(st, sh) || !tile_hd || items < 1 || ns < 1 || (ns > 1 && !partials)) return hipErrorInvalidValue;
+  const bool pad = tile_hd != sh.hd;
   const PrefillLaunch plan = plan_prefill_launch(sh, items, ns, wgs_per_cu, groups_wanted);
   const long long n_wgs = plan.n_wgs;
   if (n_wgs > 0x7fffffffLL) return hipErrorInvalidValue;
@@ -716,47 +733,64 @@ hipError_t launch_prefill(const float *q_rot, const float *kc, const float *vc, 
   const float c = scale * kLog2e;
   dim3 grid((unsigned)n_wgs);
   float *part_o = partials;
-  float *part_ml = partials ? partials + (size_t)items * sh.KV * ns * 128 * sh.hd : nullptr;
+  float *part_ml = partials ? partials + (size_t)items * sh.KV * ns * 128 * tile_hd : nullptr;
   const int groups = plan.groups;
-  const size_t pad = plan.pad;
+  const size_t lds_pad = plan.pad;
   if (plan.turns) {
     const int turns = plan.turns;
     dim3 fewer((unsigned)((n_wgs + turns - 1) / turns));
-    if (sh.hd == 64)
-      SHAINET_LAUNCH_TIMED((prefill_turns_kernel<64, 2>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, vc, out,
-                           st, sh, (int)n_wgs, c);
-    else
-      SHAINET_LAUNCH_TIMED((prefill_turns_kernel<128, 2>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, vc, out,
-                           st, sh, (int)n_wgs, c);
+#define SHAINET_LAUNCH_TURNS(HD_, PAD_)                                                                          \
+  SHAINET_LAUNCH_TIMED((prefill_turns_kernel<HD_, 2, PAD_>), fewer, dim3(512), 0, stream, before, after, q_rot, kc, \
+                       vc, out, st, sh, (int)n_wgs, c)
+    if (tile_hd == 64) {
+      if (pad)
+        SHAINET_LAUNCH_TURNS(64, true);
+      else
+        SHAINET_LAUNCH_TURNS(64, false);
+    } else {
+      if (pad)
+        SHAINET_LAUNCH_TURNS(128, true);
+      else
+        SHAINET_LAUNCH_TURNS(128, false);
+    }
+#undef SHAINET_LAUNCH_TURNS
     return hipGetLastError();
   }
   hipEvent_t main_after = ns == 1 ? after : nullptr;  // with key chunks the combine kernel ends the timed stretch
-#define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_)                                                                    \
+#define SHAINET_LAUNCH_PREFILL(HD_, SPLIT_, PAD_)                                                              \
   do {                                                                                                          \
     if (groups == 2)                                                                                            \
-      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 2>), grid, dim3(512), pad, stream, before,           \
+      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 2, PAD_>), grid, dim3(512), lds_pad, stream, before, \
                            main_after, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);                     \
     else                                                                                                        \
-      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 1>), grid, dim3(256), pad, stream, before,           \
+      SHAINET_LAUNCH_TIMED((prefill_mfma_kernel<HD_, SPLIT_, 1, PAD_>), grid, dim3(256), lds_pad, stream, before, \
                            main_after, q_rot, kc, vc, out, part_o, part_ml, st, sh, ns, c);                     \
   } while (0)
-  if (sh.hd == 64) {
-    if (ns > 1)
-      SHAINET_LAUNCH_PREFILL(64, true);
+#define SHAINET_LAUNCH_PREFILL_HD(HD_, PAD_) \
+  do {                                        \
+    if (ns > 1)                               \
+      SHAINET_LAUNCH_PREFILL(HD_, true, PAD_);   \
+    else                                      \
+      SHAINET_LAUNCH_PREFILL(HD_, false, PAD_);  \
+  } while (0)
+  if (tile_hd == 64) {
+    if (pad)
+      SHAINET_LAUNCH_PREFILL_HD(64, true);
     else
-      SHAINET_LAUNCH_PREFILL(64, false);
+      SHAINET_LAUNCH_PREFILL_HD(64, false);
   } else {
-    if (ns > 1)
-      SHAINET_LAUNCH_PREFILL(128, true);
+    if (pad)
+      SHAINET_LAUNCH_PREFILL_HD(128, true);
     else
-      SHAINET_LAUNCH_PREFILL(128, false);
+      SHAINET_LAUNCH_PREFILL_HD(128, false);
   }
+#undef SHAINET_LAUNCH_PREFILL_HD
 #undef SHAINET_LAUNCH_PREFILL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || ns == 1) return e;
   hipEvent_t none = nullptr;
   SHAINET_LAUNCH_TIMED(prefill_combine_kernel, dim3((unsigned)(items * sh.KV), 4), dim3(256), 0, stream, none, after,
-                       part_o, part_ml, out, st, sh, ns, 1.0f);  // the partials' maxima are already in log2 units
+                       part_o, part_ml, out, st, sh, ns, 1.0f, tile_hd);  // the partials' maxima are already in log2 units
   return hipGetLastError();
 }
 

@@ -139,6 +139,9 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
 // partial rows in `partials` (prefill_partial_floats) and a second kernel merges.
 int prefill_key_splits(const SeqTable &st, const Shape &sh, int items);
 size_t prefill_partial_floats(const Shape &sh, int items, int ns);
+// The head dimension the MFMA prefill kernel lays its tiles out for when the data's is hd: 64 or
+// 128, the first that holds hd (a multiple of 4); 0 when neither does.
+int prefill_tile_head_dim(int hd);
 // wgs_per_cu: 0 = default; 1..3 pads the kernel's LDS so that at most that many
 // workgroups share a compute unit (a tuning knob).
 // groups: 0 = default; 1 or 2 forces the number of wavefront groups per workgroup (a tuning knob).

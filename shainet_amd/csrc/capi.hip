@@ -1162,6 +1162,7 @@ int shainet_attn_describe_plan(int num_heads, int num_kv_heads, int head_dim, in
     if (!decode_entries(st, sh, att)) return fail(SHAINET_HIP_ERR_RUNTIME, "decode entries do not fit");
     const DecodePlan p = plan_decode(att, sh, 0);
     plan[0] = 0;
+    plan[1] = decode_tile_head_dim(head_dim);
     plan[2] = 1;
     plan[3] = 1;
     plan[5] = p.n_wgs;
@@ -1172,6 +1173,7 @@ int shainet_attn_describe_plan(int num_heads, int num_kv_heads, int head_dim, in
     const int ns = prefill_key_splits(st, sh, items);
     const PrefillLaunch p = plan_prefill_launch(sh, items, ns, 0, 0);
     plan[0] = 1;
+    plan[1] = prefill_tile_head_dim(head_dim);
     plan[2] = ns;
     plan[3] = p.groups;
     plan[4] = p.turns;

@@ -385,6 +385,12 @@ def test_config5b_long_context_batch4_decode(hip):
     (6, 2, 64, 5, 45, False),     # g = 3: virtual rows straddle rows unevenly
     (4, 4, 128, 0, 130, True),    # g = 1
     (16, 1, 64, 40, 9, False),    # g = 16
+    # head dimensions below the tile layouts' 64 and 128: padded tiles
+    (8, 2, 96, 17, 70, True),
+    (6, 2, 32, 5, 45, False),
+    (4, 4, 80, 0, 130, True),
+    (8, 4, 8, 3, 40, False),
+    (4, 1, 100, 0, 200, False),   # several row blocks per kv head
 ])
 def test_prefill_small_shapes(hip, H, KV, hd, S, T, norm):
     ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=norm, capacity=256, seed=T)
@@ -400,7 +406,8 @@ def test_prefill_key_splits(hip, ns, monkeypatch):
     # key range of every row block cut into ns chunks merged by a second kernel; with S = 0 the later
     # chunks start past the last visible key of the early rows (their partial stays at -inf)
     monkeypatch.setenv("SHAINET_HIP_PREFILL_SPLITS", str(ns))
-    for H, KV, hd, S, T, norm in [(8, 2, 64, 0, 70, False), (8, 1, 128, 100, 37, True), (6, 2, 64, 300, 130, False)]:
+    for H, KV, hd, S, T, norm in [(8, 2, 64, 0, 70, False), (8, 1, 128, 100, 37, True), (6, 2, 64, 300, 130, False),
+                                  (8, 2, 96, 200, 40, True), (4, 2, 24, 0, 150, False)]:
         ctx, cache, blocks, r = make_pair(hip, H, KV, hd, 1e6, norm=norm, capacity=512, seed=ns + T)
         if S:
             check_step(ctx, cache, blocks, r, [S])

@@ -53,6 +53,14 @@ def test_decode_and_generic_paths_are_told_apart():
     assert sa.describe_plan(32, 8, 128, [5000] * 16, [1] * 16)["path"] == sa.hip.PATH_DECODE
     assert sa.describe_plan(32, 8, 128, [5000] * 16, [8] * 16)["path"] == sa.hip.PATH_DECODE  # two entries each
     assert sa.describe_plan(32, 8, 128, [5000] * 16, [9] * 16)["path"] == sa.hip.PATH_PREFILL
-    assert sa.describe_plan(8, 4, 8, [0], [6])["path"] == sa.hip.PATH_GENERIC
+    # head dimensions between the tile layouts run in padded tiles: 8 in tiles of 64, 96 in tiles of 128
+    small = sa.describe_plan(8, 4, 8, [0], [6])
+    assert small["path"] == sa.hip.PATH_DECODE and small["head_dim"] == 64
+    assert sa.describe_plan(32, 8, 96, [0], [300])["path"] == sa.hip.PATH_PREFILL
+    assert sa.describe_plan(32, 8, 96, [0], [300])["head_dim"] == 128
+    assert sa.describe_plan(16, 4, 256, [4096], [1])["head_dim"] == 256
+    # what no tile layout holds: not a multiple of 4, or more than 16 rows x heads of head_dim above 128
+    assert sa.describe_plan(8, 4, 6, [0], [6])["path"] == sa.hip.PATH_GENERIC
+    assert sa.describe_plan(16, 4, 256, [0], [40])["path"] == sa.hip.PATH_GENERIC
     head = sa.describe_plan(32, 8, 128, [5000] * 16, [1] * 16)
     assert head["workgroups"] == 256 and head["units"] * 256 >= 16 * 8 * 313
