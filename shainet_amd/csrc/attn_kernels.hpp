@@ -190,6 +190,8 @@ struct GemvArgs {
   float *y;              // [T, N]; kGemvSwiglu: silu(x W_gate) * (x W_up)
   float *partials;       // GemvPlan::partial_floats floats when the plan has splits > 1
   unsigned *flags;       // GemvPlan::col_tiles * splits words, zero when allocated; left zero
+  unsigned *flag_set;    // null, or where partials are marked complete instead of in `flags` (the test of the give-up path)
+  int spin_limit;        // 0, or the polls after which a wait is given up (that test)
   int *error;            // device-writable int, set to 1 when a wait for partials was given up
   int T, K, N;
   int epilogue;

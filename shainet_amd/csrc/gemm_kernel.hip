@@ -68,7 +68,9 @@ struct GemmArgs {
   const float *res;  // nullable: y = res + x W
   float *partials;   // [workgroups][128 * 128]: the piece a workgroup leaves unfinished
   unsigned *flags;   // [workgroups], zero between launches
-  int *error;        // set to 1 when a wait for a flag word is given up
+  unsigned *flag_set;  // where a piece is marked complete: `flags`, or elsewhere in the test of the give-up path
+  int spin_limit;    // polls before a wait for a flag word is given up
+  int *error;        // set to 1 then
   int T, K, N, tiles_m;
   int steps;            // K steps of 32 per tile
   int group_bits;       // workgroup id -> group id & (groups - 1), place id >> group_bits
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const GemmArgs g) {
       // before the piece is marked complete
       __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
-      if (threadIdx.x == 0) __hip_atomic_store(g.flags + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (threadIdx.x == 0) __hip_atomic_store(g.flag_set + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       continue;
     }
     if (s_begin > 0) {
@@ -281,7 +283,7 @@ __global__ __launch_bounds__(256, 2) void sgemm_mfma_kernel(const GemmArgs g) {
                                  __HIP_MEMORY_SCOPE_AGENT);
             break;
           }
-          if (spins >= (1 << 21)) {  // seconds
+          if (spins >= g.spin_limit) {
             if (lane == 0) *g.error = 1;
             break;
           }
@@ -404,7 +406,8 @@ GemmPlan plan_gemm(int T, int K, int N, long long x_stride) {
 }
 
 hipError_t launch_gemm(const float *x, long long x_stride, const float *w, float *y, const float *res, float *partials,
-                       unsigned *flags, int *error, int T, int K, int N, const GemmPlan &p, hipStream_t stream) {
+                       unsigned *flags, int *error, int T, int K, int N, const GemmPlan &p, hipStream_t stream,
+                       unsigned *flag_set, int spin_limit) {
   if (!x || !w || !y || T < 1 || K < 1 || N < 1 || x_stride < K) return hipErrorInvalidValue;
   const bool aligned = !(((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)res) & 15);
   if (!p.mfma || !aligned) {
@@ -422,6 +425,8 @@ hipError_t launch_gemm(const float *x, long long x_stride, const float *w, float
   g.res = res;
   g.partials = partials;
   g.flags = flags;
+  g.flag_set = flag_set ? flag_set : flags;
+  g.spin_limit = spin_limit > 0 ? spin_limit : 1 << 21;  // polls of about a microsecond each: seconds
   g.error = error;
   g.T = T;
   g.K = K;

@@ -21,7 +21,10 @@ GemmPlan plan_gemm(int T, int K, int N, long long x_stride);
 // res are dense [T, N]; res nullable (y = res + x W; res == y is allowed).  partials, flags:
 // p.partial_floats floats and p.flag_words words (unused when those are 0); error: a word the
 // kernel sets to 1 when it gives up a wait for another workgroup's piece (y is invalid then).
+// flag_set, spin_limit: for the test of the give-up path only (marks go to flag_set, p.flag_words
+// words of their own, instead of flags, and a wait ends after spin_limit polls); null / 0 otherwise.
 hipError_t launch_gemm(const float *x, long long x_stride, const float *w, float *y, const float *res, float *partials,
-                       unsigned *flags, int *error, int T, int K, int N, const GemmPlan &p, hipStream_t stream);
+                       unsigned *flags, int *error, int T, int K, int N, const GemmPlan &p, hipStream_t stream,
+                       unsigned *flag_set = nullptr, int spin_limit = 0);
 
 }  // namespace shainet

@@ -266,7 +266,9 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   __syncthreads();
   unsigned *flags = a.flags + (long long)blockIdx.x * splits;
   if ((int)blockIdx.y != splits - 1) {
-    if (threadIdx.x == 0) __hip_atomic_store(flags + blockIdx.y, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0)
+      __hip_atomic_store((a.flag_set ? a.flag_set : a.flags) + (long long)blockIdx.x * splits + blockIdx.y, 1u,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   // the others have lower indices, were started before this workgroup and wait for nobody
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
           __hip_atomic_store(flags + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
-      if (spins >= (1 << 21)) {  // seconds
+      if (spins >= (a.spin_limit > 0 ? a.spin_limit : 1 << 21)) {  // (by default: seconds)
         if (lane == 0) *a.error = 1;
         break;
       }

@@ -80,6 +80,10 @@ struct Projector {
   // split products: a word per partial that says when it is complete (zero between launches)
   unsigned *flags = nullptr;
   size_t flags_cap = 0;
+  // SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS (read when the flag words are first allocated): the marks
+  // go to a second set of words nobody reads and waits end after 2000 polls, so that the report
+  // of a given-up wait can be exercised without hanging anything
+  bool lose_marks = false;
   // where the split products' kernels report a given-up wait: the owner's pinned host word
   int *error = nullptr;
   // returns a SHAINET_HIP_* status; the message is left for shainet_hip_last_error

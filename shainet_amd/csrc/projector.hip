@@ -67,11 +67,13 @@ void DevF::release() {
 // launches of one projector follow each other on one stream.
 int Projector::reserve_flags(size_t n_flags, hipStream_t stream) {
   if (n_flags <= flags_cap) return SHAINET_HIP_OK;
+  if (!flags) lose_marks = getenv("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS") != nullptr;
   size_t want = flags_cap ? flags_cap : 4096;
   while (want < n_flags) want *= 2;
   unsigned *np = nullptr;
-  if (hipMalloc((void **)&np, want * sizeof(unsigned)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
-  if (hipMemsetAsync(np, 0, want * sizeof(unsigned), stream) != hipSuccess) {
+  // (twice the words: the second half is where the marks go in the test of the give-up path)
+  if (hipMalloc((void **)&np, 2 * want * sizeof(unsigned)) != hipSuccess) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
+  if (hipMemsetAsync(np, 0, 2 * want * sizeof(unsigned), stream) != hipSuccess) {
     (void)hipFree(np);
     return llama_fail(SHAINET_HIP_ERR_RUNTIME, "hipMemsetAsync(flags) failed");
   }
@@ -88,7 +90,8 @@ int Projector::gemm(const float *x, long long x_stride, const float *w, float *y
   if (!scratch.reserve(p.partial_floats)) return llama_fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
   if (int rc = reserve_flags(p.flag_words, stream)) return rc;
   if (p.flag_words && !error) return llama_fail(SHAINET_HIP_ERR_RUNTIME, "the projector has no error word");
-  hipError_t e = launch_gemm(x, x_stride, w, y, res, scratch.p, flags, error, T, K, N, p, stream);
+  hipError_t e = launch_gemm(x, x_stride, w, y, res, scratch.p, flags, error, T, K, N, p, stream,
+                             lose_marks ? flags + flags_cap : nullptr, lose_marks ? 2000 : 0);
   if (e != hipSuccess) return llama_fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemm launch: ") + hipGetErrorString(e));
   return SHAINET_HIP_OK;
 }
@@ -126,6 +129,8 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.y = y;
     a.partials = scratch.p;
     a.flags = flags;
+    a.flag_set = lose_marks ? flags + flags_cap : nullptr;
+    a.spin_limit = lose_marks ? 2000 : 0;
     a.error = error;
     a.T = T;
     a.K = K;

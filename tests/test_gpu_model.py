@@ -193,6 +193,37 @@ def test_matmul_matches_oracle(hip, T, K, N, res, stride):
     assert torch.equal(got, again)
 
 
+def test_matmul_reports_a_given_up_wait(hip):
+    """The split products wait, bounded, for the partial sums of other workgroups (the split GEMV up to
+    16 rows, the MFMA product where workgroups share a tile).  Forced from the host in a child
+    process: the completion marks go where nobody looks and a wait ends after 2000 polls; the call
+    after such a launch on the same stream says so and does nothing else."""
+    import subprocess
+    import sys
+
+    code = """
+import torch
+from shainet_amd import hip
+for T, K, N in ((5, 2048, 2048), (700, 512, 640)):
+    x = torch.randn((T, K), device="cuda"); w = torch.randn((K, N), device="cuda")
+    hip.matmul(x, w); torch.cuda.synchronize()
+    try:
+        hip.matmul(x, w)
+        print("no report", T)
+    except hip.HipError as e:
+        print("reported", T, e)
+    torch.cuda.synchronize()
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS="1", PYTHONPATH=root)
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.count("reported") == 2 and done.stdout.count("gave up waiting") == 2, done.stdout + done.stderr[-2000:]
+    env.pop("SHAINET_HIP_TEST_LOSE_PARTIAL_MARKS")
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and done.stdout.count("no report") == 2, done.stdout + done.stderr[-2000:]
+
+
 def test_matmul_full_tiles_llama1b_prefill_shapes(hip):
     # 512 rows of the four products of a Llama-3.2-1B block against torch in fp64 (the oracle's scalar
     # loop would take minutes here; it is pinned against the same fp64 product in tests/test_oracle_pins.py)
