@@ -277,7 +277,9 @@ def describe_plan(num_heads, num_kv_heads, head_dim, start_pos, new_tokens):
     sp, nt = (C.c_int * n)(*start_pos), (C.c_int * n)(*new_tokens)
     plan = (C.c_int * 8)()
     _check(lib().shainet_attn_describe_plan(num_heads, num_kv_heads, head_dim, n, sp, nt, plan))
-    return dict(zip(PLAN_FIELDS, (int(v) for v in plan)))
+    d = dict(zip(PLAN_FIELDS, (int(v) for v in plan)))
+    d["padded"] = d["head_dim"] != head_dim   # the tiles are laid out for a larger head_dim than the data's
+    return d
 
 
 def matmul(x, w, res=None, out=None, stream=None):

@@ -1,6 +1,7 @@
 """The prefill launches whose parity the GPU suite checks at full size, each with the kernel
 instantiation the library's own planner picks for it: (head_dim, key chunks merged by the
-combine kernel?, wavefront groups, row blocks a workgroup takes in turn).
+combine kernel?, wavefront groups, row blocks a workgroup takes in turn), and `+ (True,)` for the
+instantiations that run a smaller head_dim in padded tiles.
 
 tests/test_gpu_parity.py runs every case against the oracle on all rows with no tuning
 variable set and asserts that the planner's choice is the instantiation named here;
@@ -22,6 +23,11 @@ CASES = [
     ("qwen3_8b_prefill_t3072", 32, 8, 128, True, 0, 3072, (128, False, 2, 3)),
     ("qwen3_8b_prefill_t2560", 32, 8, 128, True, 0, 2560, (128, False, 2, 0)),
     ("qwen3_8b_prefill_t4096", 32, 8, 128, True, 0, 4096, (128, False, 1, 0)),
+    # head dims below the tile layouts (padded tiles): Phi-3-mini's heads at the bench's size, and smaller ones
+    ("phi3_hd96_prefill_t2048", 32, 32, 96, False, 0, 2048, (128, False, 2, 2, True)),
+    ("hd96_chunked_prefill_t256_on_8192", 16, 4, 96, True, 8192, 256, (128, True, 2, 0, True)),
+    ("hd48_prefill_t8192", 16, 8, 48, False, 0, 8192, (64, False, 1, 0, True)),
+    ("hd32_prefill_t1024", 32, 8, 32, True, 0, 1024, (64, True, 2, 0, True)),
 ]
 
 # The prefill shapes of the benchmark configurations (BASELINE.json configs[3] and configs[4](a)):
@@ -35,4 +41,5 @@ BASELINE_PREFILL_SHAPES = [
 
 def instantiation(plan):
     """The kernel instantiation of a plan dict from shainet_amd.describe_plan."""
-    return (plan["head_dim"], plan["key_chunks"] > 1, plan["groups"], plan["turns"])
+    inst = (plan["head_dim"], plan["key_chunks"] > 1, plan["groups"], plan["turns"])
+    return inst + (True,) if plan.get("padded") else inst

@@ -36,7 +36,10 @@ def test_bench_prefill_workloads_are_cases():
 
 
 def test_every_reachable_instantiation_is_covered():
-    covered = {inst for *_, inst in pc.CASES}
+    # (the instantiations for padded tiles, a fifth element in the table, are the same code with the
+    # head_dim of the data as a run-time value; the table holds four of them, both tile widths, with
+    # and without key chunks, turns and one workgroup per block, and this sweep does not enumerate them)
+    covered = {inst for *_, inst in pc.CASES if len(inst) == 4}
     seen = set()
     for hd, KV, g in itertools.product((64, 128), (1, 2, 4, 8), (1, 2, 4, 8)):
         for S in (0, 1000, 4096, 16384, 32768):
