@@ -208,6 +208,11 @@ struct GemvPlan {
 // head_dim: kGemvQkvPrep only (a column tile must hold whole heads)
 GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim = 0);
 hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
+// The same product for one row of x against weights kept transposed (a.w: [N, K], or [2N, K] =
+// gate | up for kGemvSwiglu): a wavefront per output, nothing shared between wavefronts.
+// gemvt_takes: what it serves (one row; K 1024, 2048, 4096, or 8192 without norm and SwiGLU).
+bool gemvt_takes(int T, int K, int N, int epilogue, bool norm);
+hipError_t launch_gemvt(const GemvArgs &a, hipStream_t stream);
 
 // A pinned host int per context (block, model) that its kernels set when they give up a
 // bounded wait for other workgroups (null when it cannot be allocated); check_error_word,

@@ -288,7 +288,48 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const float *__restrict
   orow[i + half] = (float)(x1 * c + x0 * s);
 }
 
+// 32 x 32 tiles through LDS: coalesced on both sides
+__global__ __launch_bounds__(256) void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int rows,
+                                                        int cols) {
+  __shared__ float tile[32][33];
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int i = ty; i < 32; i += 8)
+    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = src[(long long)(r0 + i) * cols + c0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8)
+    if (c0 + i < cols && r0 + tx < rows) dst[(long long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+__global__ __launch_bounds__(256) void transposed_differ_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                                int rows, int cols, int *__restrict__ differ) {
+  __shared__ unsigned tile[32][33];
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int i = ty; i < 32; i += 8)
+    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = __float_as_uint(a[(long long)(r0 + i) * cols + c0 + tx]);
+  __syncthreads();
+  bool bad = false;
+  for (int i = ty; i < 32; i += 8)
+    if (c0 + i < cols && r0 + tx < rows) bad = bad || __float_as_uint(b[(long long)(c0 + i) * rows + r0 + tx]) != tile[tx][i];
+  if (bad) *differ = 1;
+}
+
 }  // namespace
+
+hipError_t launch_transposed_differ(const float *a, const float *b, int rows, int cols, int *differ, hipStream_t stream) {
+  if (!a || !b || !differ || rows < 1 || cols < 1 || (rows + 31) / 32 > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(transposed_differ_kernel, dim3((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32)), dim3(256),
+                     0, stream, a, b, rows, cols, differ);
+  return hipGetLastError();
+}
+
+hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream) {
+  if (!src || !dst || rows < 1 || cols < 1 || (rows + 31) / 32 > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32)), dim3(256), 0,
+                     stream, src, dst, rows, cols);
+  return hipGetLastError();
+}
 
 hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
                           double eps, hipStream_t stream) {

@@ -10,6 +10,11 @@ namespace shainet {
 // the rows of x are x_stride floats apart, those of out are dense
 hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
                           double eps, hipStream_t stream);
+// dst[c, r] = src[r, c]: src is [rows, cols], dst [cols, rows], both dense
+hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream);
+// *differ (a device int the caller has set to 0) becomes 1 when a [rows, cols] is not, bit for bit,
+// the transpose of b [cols, rows]
+hipError_t launch_transposed_differ(const float *a, const float *b, int rows, int cols, int *differ, hipStream_t stream);
 // out = a + b, n floats
 hipError_t launch_add(const float *a, const float *b, float *out, long long n, hipStream_t stream);
 // hidden[r, j] = silu(gate_up[r, j]) * gate_up[r, ff + j];  gate_up is [rows, 2*ff]

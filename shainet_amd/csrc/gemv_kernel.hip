@@ -20,6 +20,7 @@
 #include "prep_math.hpp"
 
 #include <math.h>
+#include <stdint.h>
 #include <stdlib.h>
 
 namespace shainet {
@@ -351,6 +352,104 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
   }
 }
 
+
+// ---- one row of x against weights kept transposed: wt [N, K] (row n = column n of W) --------
+// Every output element is one contiguous row of wt, so a wavefront owns whole outputs: it reads
+// a row with KV4 16-byte loads per lane, all in flight at once, multiplies by the x values it
+// keeps in registers and adds up across its lanes.  Nothing crosses wavefronts: no partial sums
+// in memory, no flag words, no wait, no LDS, and a launch ends when its rows have streamed (a
+// 2048 x 2048 product: 4.8 us back to back against 8.8 us for the split product above).  What it
+// costs is the second copy of the matrix.  NACC = 2: the SwiGLU epilogue; the wavefront reads row
+// n (gate) and row N + n (up).  K = 256 KV4.  The RMSNorm prologue is done by every wavefront for
+// itself from the x values it holds (fp64 as rms_norm.cr:18-37; another order of the additions
+// than the split product's).
+// SP = 2: two wavefronts share an output, half a row each (K = 512 KV4), and add up through LDS:
+// rows of 8192 values, which one wavefront could only hold with a single wavefront per SIMD
+// (no norm prologue then, and NACC = 1).
+template <int KV4, int NACC, int SP>
+__global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
+  __shared__ float half_s[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * (4 / SP) + wave / SP;  // the output this wavefront owns (or shares)
+  const int seg = wave % SP;
+  const int N = a.N;
+  constexpr int K = 256 * KV4 * SP;
+  // (with SP = 2, N is even: launch_gemvt sees to it, so both wavefronts of a pair are in or out)
+  if (n >= N) return;
+  f32x4 w[NACC][KV4];
+#pragma unroll
+  for (int c = 0; c < NACC; ++c) {
+    const float *row = a.w + ((long long)c * N + n) * K + seg * (256 * KV4) + 4 * lane;
+#pragma unroll
+    for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
+  }
+  // x: up to 2048 values stay in registers; longer rows are read again, eight 16-byte pieces at
+  // a time (from the L2), where they are used, the registers being needed for the row of wt
+  constexpr int XC = KV4 < 8 ? KV4 : 8;
+  const float *xp = a.x + seg * (256 * KV4) + 4 * lane;
+  double rms = 1.0;  // 1 / the root mean square
+  if (a.norm) {
+    double sq = 0.0;
+#pragma unroll
+    for (int c0 = 0; c0 < KV4; c0 += XC) {
+      f32x4 xv[XC];
+#pragma unroll
+      for (int i = 0; i < XC; ++i) xv[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
+#pragma unroll
+      for (int i = 0; i < XC; ++i) {
+        sq += (double)xv[i].x * (double)xv[i].x + (double)xv[i].y * (double)xv[i].y;
+        sq += (double)xv[i].z * (double)xv[i].z + (double)xv[i].w * (double)xv[i].w;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+    // (x / rms as x * (1 / rms): every wavefront norms the whole row for itself, and a division
+    // per element, eight wavefronts' worth per SIMD, cost 5 of the 26 us of a 2048 -> 2 x 8192 product)
+    rms = 1.0 / sqrt(sq / (double)K + a.eps);
+  }
+  f32x4 acc[NACC];
+#pragma unroll
+  for (int c = 0; c < NACC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c0 = 0; c0 < KV4; c0 += XC) {
+    f32x4 xv[XC];
+#pragma unroll
+    for (int i = 0; i < XC; ++i) xv[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
+    if (a.norm) {
+#pragma unroll
+      for (int i = 0; i < XC; ++i) {
+        f32x4 g = {1.f, 1.f, 1.f, 1.f};
+        if (a.gamma) g = *(const f32x4 *)(a.gamma + 4 * lane + 256 * (c0 + i));
+        xv[i] = f32x4{(float)(((double)xv[i].x * rms) * (double)g.x), (float)(((double)xv[i].y * rms) * (double)g.y),
+                      (float)(((double)xv[i].z * rms) * (double)g.z), (float)(((double)xv[i].w * rms) * (double)g.w)};
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NACC; ++c)
+#pragma unroll
+      for (int i = 0; i < XC; ++i) acc[c] += w[c][c0 + i] * xv[i];
+  }
+  float s[NACC];
+#pragma unroll
+  for (int c = 0; c < NACC; ++c) {
+    s[c] = (acc[c].x + acc[c].y) + (acc[c].z + acc[c].w);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s[c] += __shfl_xor(s[c], o);
+  }
+  if constexpr (SP == 2) {
+    if (lane == 0) half_s[wave] = s[0];
+    __syncthreads();
+    if (seg) return;
+    s[0] = half_s[wave] + half_s[wave + 1];
+  }
+  if (lane == 0) {
+    float v = s[0];
+    if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
+    if (a.epilogue == kGemvResidual) v = (float)((double)a.res[n] + (double)s[0]);
+    a.y[n] = v;
+  }
+}
+
 }  // namespace
 
 GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim) {
@@ -434,6 +533,41 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
     SHAINET_LAUNCH_GEMV_T(2, 4, false);
 #undef SHAINET_LAUNCH_GEMV_T
 #undef SHAINET_LAUNCH_GEMV
+  return hipGetLastError();
+}
+
+bool gemvt_takes(int T, int K, int N, int epilogue, bool norm) {
+  if (T != 1 || N < 1) return false;
+  // rows of 8192: two wavefronts per output, which leaves out the norm prologue and SwiGLU
+  if (K == 8192) return !norm && !(N & 1) && (epilogue == kGemvPlain || epilogue == kGemvResidual);
+  if (K != 1024 && K != 2048 && K != 4096) return false;
+  return epilogue == kGemvPlain || epilogue == kGemvResidual || epilogue == kGemvSwiglu;
+}
+
+hipError_t launch_gemvt(const GemvArgs &args, hipStream_t stream) {
+  GemvArgs a = args;
+  if (!gemvt_takes(a.T, a.K, a.N, a.epilogue, a.norm != 0) || !a.x || !a.w || !a.y) return hipErrorInvalidValue;
+  if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
+  if (((uintptr_t)a.x | (uintptr_t)a.w | (uintptr_t)a.gamma) & 15) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((a.N + 3) / 4));
+  const bool two = a.epilogue == kGemvSwiglu;
+#define SHAINET_LAUNCH_GEMVT(KV4_)                                                     \
+  do {                                                                                 \
+    if (two)                                                                           \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 2, 1>), grid, dim3(256), 0, stream, a);   \
+    else                                                                               \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 1, 1>), grid, dim3(256), 0, stream, a);   \
+  } while (0)
+  switch (a.K) {
+    case 1024: SHAINET_LAUNCH_GEMVT(4); break;
+    case 2048: SHAINET_LAUNCH_GEMVT(8); break;
+    case 4096: SHAINET_LAUNCH_GEMVT(16); break;
+    default:  // 8192: two wavefronts per output
+      if (two || a.norm || (a.N & 1)) return hipErrorInvalidValue;
+      hipLaunchKernelGGL((gemvt_kernel<16, 1, 2>), dim3((unsigned)(a.N / 2)), dim3(256), 0, stream, a);
+      break;
+  }
+#undef SHAINET_LAUNCH_GEMVT
   return hipGetLastError();
 }
 

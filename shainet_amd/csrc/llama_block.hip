@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <new>
@@ -38,6 +39,10 @@ struct shainet_llama_attn {
   bool has_rope_freqs = false, has_q_norm = false, has_k_norm = false, has_bq = false, has_bk = false, has_bv = false;
   bool params_dirty = true;  // setters may run after construction (hf_loader.cr:319-373)
   float *w_qkv = nullptr, *w_o = nullptr;  // device, [in, out]; w_q | w_k | w_v side by side in one matrix
+  // w_o once more, transposed ([d_model, q_dim]), for the product of a single row (launch_gemvt):
+  // made on the device when such a call first needs it, made again after the weights change
+  float *w_o_t = nullptr;
+  bool w_o_t_stale = true;
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
   shainet_kv_cache *scratch_cache = nullptr;  // rows of a no-cache forward call; empty between calls
@@ -152,6 +157,7 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     post.epilogue = kGemvResidual;
     post.res = residual;
   }
+  if (gemvt_takes(T, l->q_dim, l->d_model, post.epilogue, false)) post.w_t = transposed_twin(&l->w_o_t, &l->w_o_t_stale, l->w_o, l->q_dim, l->d_model, stream);
   return l->proj.project(l->attn.p, l->q_dim, l->w_o, out, T, l->q_dim, l->d_model, stream, post);  // 298
 }
 
@@ -190,7 +196,7 @@ int shainet_llama_attn_destroy(shainet_llama_attn *l) {
   if (!l) return SHAINET_HIP_OK;
   drop_context(l);
   l->proj.release();
-  for (float *p : {l->w_qkv, l->w_o})
+  for (float *p : {l->w_qkv, l->w_o, l->w_o_t})
     if (p) (void)hipFree(p);
   for (DevF *b : {&l->x, &l->qkv, &l->attn, &l->out}) b->release();
   l->x_pin.release();
@@ -234,6 +240,7 @@ int shainet_llama_attn_set_weights(shainet_llama_attn *l, const float *w_q, cons
   const int widths[3] = {l->q_dim, l->kv_dim, l->kv_dim};
   int rc = upload_side_by_side(&l->w_qkv, mats, widths, 3, l->d_model);
   if (!rc) rc = upload_floats(&l->w_o, w_o, (size_t)l->q_dim * l->d_model);
+  l->w_o_t_stale = true;
   return rc;
 }
 
@@ -289,6 +296,8 @@ struct shainet_llama_block {
   double eps = 1e-6;                                // RMSNorm eps of @norm1 / @norm2 (llama_block.cr:93-94)
   float *norm1 = nullptr, *norm2 = nullptr;         // device gamma [d_model]; null = ones (rms_norm.cr:10)
   float *gate_up = nullptr, *down = nullptr;        // device [d_model, 2*ff] (gate | up) and [ff, d_model]
+  float *gate_up_t = nullptr, *down_t = nullptr;    // the same transposed ([2*ff, d_model], [d_model, ff]), like w_o_t
+  bool gate_up_t_stale = true, down_t_stale = true;
   DevF x, h, hidden, out;
   PinnedF x_pin, out_pin;  // host-pointer calls stage their rows here
 };
@@ -317,11 +326,13 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
   gate.gamma = b->norm2;
   gate.eps = b->eps;
   gate.epilogue = kGemvSwiglu;
+  if (gemvt_takes(T, d, ff, gate.epilogue, true)) gate.w_t = transposed_twin(&b->gate_up_t, &b->gate_up_t_stale, b->gate_up, d, 2 * ff, stream);
   if ((rc = l->proj.project(b->h.p, d, b->gate_up, b->hidden.p, T, d, ff, stream, gate))) return rc;
   // out = h + hidden * down_proj
   Fused down;
   down.epilogue = kGemvResidual;
   down.res = b->h.p;
+  if (gemvt_takes(T, ff, d, down.epilogue, false)) down.w_t = transposed_twin(&b->down_t, &b->down_t_stale, b->down, ff, d, stream);
   return l->proj.project(b->hidden.p, ff, b->down, out, T, ff, d, stream, down);
 }
 
@@ -345,6 +356,8 @@ int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out) 
       *w.p = nullptr;
       return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
     }
+  // (whoever asks for the buffers is about to write the weights: the transposed copies are made again)
+  l->w_o_t_stale = b->gate_up_t_stale = b->down_t_stale = true;
   *out = LlamaBlockBuffers{l->w_qkv, l->w_o, b->gate_up, b->down, b->norm1, b->norm2,
                            b->d_model, l->q_dim, l->kv_dim, b->ff_hidden};
   return SHAINET_HIP_OK;
@@ -449,7 +462,7 @@ int shainet_llama_block_create(shainet_llama_block **out, int d_model, int num_h
 int shainet_llama_block_destroy(shainet_llama_block *b) {
   if (!b) return SHAINET_HIP_OK;
   shainet_llama_attn_destroy(b->attn);
-  for (float *p : {b->norm1, b->norm2, b->gate_up, b->down})
+  for (float *p : {b->norm1, b->norm2, b->gate_up, b->down, b->gate_up_t, b->down_t})
     if (p) (void)hipFree(p);
   for (DevF *f : {&b->x, &b->h, &b->hidden, &b->out}) f->release();
   b->x_pin.release();
@@ -484,6 +497,7 @@ int shainet_llama_block_set_ffn(shainet_llama_block *b, const float *gate, const
   const int widths[2] = {b->ff_hidden, b->ff_hidden};
   int rc = upload_side_by_side(&b->gate_up, mats, widths, 2, b->d_model);
   if (!rc) rc = upload_floats(&b->down, down, (size_t)b->ff_hidden * b->d_model);
+  b->gate_up_t_stale = b->down_t_stale = true;
   return rc;
 }
 

@@ -68,6 +68,9 @@ struct Fused {
   const float *gamma = nullptr;
   double eps = 0.0;
   const GemvPrep *prep = nullptr;  // kGemvQkvPrep: where the head rows go (y may be null); at most 16 rows
+  // the same weights transposed ([N, K]; kGemvSwiglu: [2N, K]) or null: one row of x then takes the
+  // product that gives a wavefront whole outputs (launch_gemvt) where its shapes allow
+  const float *w_t = nullptr;
 };
 
 // y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows
@@ -104,5 +107,12 @@ int upload_floats(float **dst, const float *src, size_t n);
 int upload_side_by_side(float **dst, const float *const *mats, const int *widths, int count, int rows);
 
 int llama_fail(int code, const std::string &msg);
+
+// Second copies of weight matrices, transposed, for the product of a single row (launch_gemvt).
+// SHAINET_HIP_NO_TRANSPOSED_WEIGHTS turns them off.  transposed_twin: *twin = src ([rows, cols] on
+// the device) transposed, allocated on first use and made again when *stale; returns the twin, or
+// null when they are turned off or there is no memory for one (the caller then goes without).
+bool transposed_twins_wanted();
+const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream);
 
 }  // namespace shainet

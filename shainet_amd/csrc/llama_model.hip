@@ -69,6 +69,12 @@ struct shainet_llama_model {
   float *final_norm = nullptr;  // device [d_model]; has_final_norm says whether the step exists (@final_norm)
   bool has_final_norm = false;
   float *lm_head = nullptr;     // device [d_model, vocab]
+  // lm_head transposed ([vocab, d_model]) for the product of a single row: the embedding table
+  // itself where the two are tied (compared on the device, bit for bit, the first time it is
+  // needed), else a copy of its own
+  const float *lm_head_t = nullptr;
+  float *lm_head_t_own = nullptr;
+  bool lm_head_t_stale = true;
   float *lm_bias = nullptr;     // device [vocab] or null
   hipStream_t stream = nullptr;
   int *error = nullptr;  // pinned host word: set by any kernel of the model that gave up a bounded wait
@@ -105,6 +111,7 @@ int shainet_llama_model_buffers(shainet_llama_model *m, LlamaModelBuffers *out) 
       return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
     }
   m->has_final_norm = true;
+  m->lm_head_t_stale = true;  // (whoever asks for the buffers is about to write them)
   if (m->lm_bias) (void)hipFree(m->lm_bias);  // the loader's output bias is all zeros (hf_loader.cr:404)
   m->lm_bias = nullptr;
   *out = LlamaModelBuffers{m->embedding, m->final_norm, m->lm_head};
@@ -112,6 +119,33 @@ int shainet_llama_model_buffers(shainet_llama_model *m, LlamaModelBuffers *out) 
 }
 
 namespace {
+
+// lm_head transposed, or null (see the struct).  The comparison with the embedding table waits
+// for the stream once, when the weights are new.
+const float *lm_head_twin(shainet_llama_model *m) {
+  if (!transposed_twins_wanted() || !m->lm_head) return nullptr;
+  if (!m->lm_head_t_stale) return m->lm_head_t;
+  m->lm_head_t = nullptr;
+  m->lm_head_t_stale = false;
+  if (m->embedding) {
+    int *differ = nullptr, host = 1;
+    if (hipMalloc((void **)&differ, sizeof(int)) == hipSuccess) {
+      bool ok = hipMemsetAsync(differ, 0, sizeof(int), m->stream) == hipSuccess &&
+                launch_transposed_differ(m->lm_head, m->embedding, m->d_model, m->vocab, differ, m->stream) == hipSuccess &&
+                hipMemcpyAsync(&host, differ, sizeof(int), hipMemcpyDeviceToHost, m->stream) == hipSuccess &&
+                hipStreamSynchronize(m->stream) == hipSuccess;
+      (void)hipFree(differ);
+      if (ok && host == 0) {
+        if (m->lm_head_t_own) (void)hipFree(m->lm_head_t_own);
+        m->lm_head_t_own = nullptr;
+        return m->lm_head_t = m->embedding;
+      }
+    }
+    (void)hipGetLastError();
+  }
+  bool stale = true;
+  return m->lm_head_t = transposed_twin(&m->lm_head_t_own, &stale, m->lm_head, m->d_model, m->vocab, m->stream);
+}
 
 int reserve_ints(int **p, size_t *cap, size_t n) {
   if (n <= *cap) return SHAINET_HIP_OK;
@@ -300,6 +334,7 @@ int run_device_tokens(shainet_llama_model *m, const int *d_tokens, int T, bool n
   fin.norm = m->has_final_norm;
   fin.gamma = m->final_norm;
   fin.eps = m->eps;
+  if (gemvt_takes(1, d, m->vocab, fin.epilogue, fin.norm)) fin.w_t = lm_head_twin(m);
   if ((rc = m->proj.project(last, d, m->lm_head, m->logits.p, 1, d, m->vocab, m->stream, fin))) return rc;
   if (m->lm_bias) {
     e = launch_add_bias_row(m->logits.p, m->lm_bias, m->vocab, m->stream);
@@ -342,7 +377,7 @@ int shainet_llama_model_create(shainet_llama_model **out, int vocab, int d_model
 int shainet_llama_model_destroy(shainet_llama_model *m) {
   if (!m) return SHAINET_HIP_OK;
   for (shainet_llama_block *b : m->blocks) shainet_llama_block_destroy(b);
-  for (float *p : {m->embedding, m->final_norm, m->lm_head, m->lm_bias, m->d_vals})
+  for (float *p : {m->embedding, m->final_norm, m->lm_head, m->lm_bias, m->d_vals, m->lm_head_t_own})
     if (p) (void)hipFree(p);
   if (m->d_tokens) (void)hipFree(m->d_tokens);
   if (m->d_ids) (void)hipFree(m->d_ids);
@@ -367,6 +402,7 @@ shainet_llama_block *shainet_llama_model_block(shainet_llama_model *m, int i) {
 int shainet_llama_model_set_embedding(shainet_llama_model *m, const float *table) {
   if (!m || !table) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  m->lm_head_t_stale = true;
   return upload_floats(&m->embedding, table, (size_t)m->vocab * m->d_model);
 }
 
@@ -381,6 +417,7 @@ int shainet_llama_model_set_final_norm(shainet_llama_model *m, const float *gamm
 int shainet_llama_model_set_lm_head(shainet_llama_model *m, const float *w, const float *bias) {
   if (!m || !w) return fail(SHAINET_HIP_ERR_ARGUMENT, "null argument");
   if (!shainet_hip_available()) return fail(SHAINET_HIP_ERR_RUNTIME, "no gfx950 device available");
+  m->lm_head_t_stale = true;
   int rc = upload_floats(&m->lm_head, w, (size_t)m->d_model * m->vocab);
   if (rc) return rc;
   if (bias) return upload_floats(&m->lm_bias, bias, (size_t)m->vocab);

@@ -1,4 +1,5 @@
 // Row-major projections on the device and small upload helpers.
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -63,6 +64,32 @@ void DevF::release() {
   cap = 0;
 }
 
+// SHAINET_HIP_NO_TRANSPOSED_WEIGHTS: no second, transposed copy of W_o, gate | up and down (the
+// products of a single row then run as the split GEMV over the [in, out] matrices, like the rest)
+bool transposed_twins_wanted() {
+  static const bool wanted = getenv("SHAINET_HIP_NO_TRANSPOSED_WEIGHTS") == nullptr;
+  return wanted;
+}
+
+// *twin = src transposed (src: [rows, cols] on the device), allocated on first use.  Returns the
+// twin, or null when there is no memory for it (the caller then goes without).
+const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream) {
+  if (!transposed_twins_wanted() || !src) return nullptr;
+  if (!*twin) {
+    if (hipMalloc((void **)twin, (size_t)rows * cols * sizeof(float)) != hipSuccess) {
+      (void)hipGetLastError();
+      *twin = nullptr;
+      return nullptr;
+    }
+    *stale = true;
+  }
+  if (*stale) {
+    if (launch_transpose(src, *twin, rows, cols, stream) != hipSuccess) return nullptr;
+    *stale = false;
+  }
+  return *twin;
+}
+
 // The flag words are shared by all kernels of this projector: each leaves them zero, and the
 // launches of one projector follow each other on one stream.
 int Projector::reserve_flags(size_t n_flags, hipStream_t stream) {
@@ -101,6 +128,25 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
   const bool swiglu = f.epilogue == kGemvSwiglu;
   if (f.epilogue == kGemvQkvPrep && (!f.prep || T > 16 || (N & 3)))
     return llama_fail(SHAINET_HIP_ERR_ARGUMENT, "the fused q | k | v epilogue takes at most 16 rows");
+  if (f.w_t && gemvt_takes(T, K, N, f.epilogue, f.norm) && !(((uintptr_t)x | (uintptr_t)f.gamma) & 15)) {
+    GemvArgs a = {};
+    a.x = x;
+    a.x_stride = x_stride;
+    a.norm = f.norm ? 1 : 0;
+    a.gamma = f.gamma;
+    a.eps = f.eps;
+    a.w = f.w_t;
+    a.res = f.res;
+    a.y = y;
+    a.T = T;
+    a.K = K;
+    a.N = N;
+    a.epilogue = f.epilogue;
+    hipError_t e = launch_gemvt(a, stream);
+    if (e != hipSuccess)
+      return llama_fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemv launch: ") + hipGetErrorString(e));
+    return SHAINET_HIP_OK;
+  }
   if (T <= 16 && (N & 3) == 0) {
     const float *xin = x;
     long long xs = x_stride;

@@ -11,7 +11,8 @@ pytestmark = pytest.mark.gpu
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SUBSET = ("decode_random_ragged or few_new_rows or prefill_random_shapes or prefill_small_shapes or prefill_key_splits "
-          "or every_small_row_count or block_forward_cached_matches or decode_every_length or two_contexts")
+          "or every_small_row_count or block_forward_cached_matches or decode_every_length or two_contexts "
+          "or single_row_products")
 
 SETTINGS = [
     {"SHAINET_HIP_DECODE_NO_ROTATE": "1"},                      # every workgroup walks its segments from their first tile
@@ -24,6 +25,7 @@ SETTINGS = [
     {"SHAINET_HIP_PREFILL_GROUPS": "1", "SHAINET_HIP_PREFILL_NO_TURNS": "1"},
     {"SHAINET_HIP_PREFILL_GROUPS": "2", "SHAINET_HIP_PREFILL_WGS_PER_CU": "2"},
     {"SHAINET_HIP_NO_FUSED_PREP": "1"},                         # q | k | v product without the prep epilogue
+    {"SHAINET_HIP_NO_TRANSPOSED_WEIGHTS": "1"},                 # one-row products over the [in, out] matrices only
 ]
 
 

@@ -454,6 +454,53 @@ def test_long_generation_across_cache_growth_equals_one_prefill(hip):
     np.testing.assert_array_equal(m.logits(), last)
 
 
+@pytest.mark.parametrize("tied", [True, False])
+def test_single_row_products_over_transposed_weights(hip, tied):
+    """One-token runs of a model whose shapes the transposed-weight product serves (W_o and gate | up
+    with K = 1024, down with K = 4096, lm_head with K = 1024): a wavefront per output over second,
+    transposed copies of the matrices, made on the device at the first such run; lm_head's is the
+    embedding table itself when the two are tied (compared on the device), a copy otherwise.
+    Against the oracle, and against the same tokens run as one prompt (MFMA products, no such copies);
+    then new weights in one block: the copies must follow."""
+    r = np.random.default_rng(5)
+    V, d, L, H, KV, ff = 700, 1024, 2, 8, 2, 4096
+    hd = d // H
+    cfg = {"vocab_size": V, "hidden_size": d, "num_hidden_layers": L, "num_attention_heads": H, "num_key_value_heads": KV,
+           "intermediate_size": ff, "rms_norm_eps": 1e-5, "rope_theta": 1e4}
+    g = lambda *sh: (r.standard_normal(sh) / np.sqrt(sh[0])).astype(np.float32)
+    embed = (0.5 * r.standard_normal((V, d))).astype(np.float32)
+    w = {"cfg": cfg, "embed": embed, "final_norm": (1 + 0.1 * r.standard_normal(d)).astype(np.float32),
+         "lm_head": np.ascontiguousarray(embed.T) if tied else g(d, V), "layers": []}
+    for _ in range(L):
+        w["layers"].append({"w_q": g(d, H * hd), "w_k": g(d, KV * hd), "w_v": g(d, KV * hd), "w_o": g(H * hd, d),
+                            "gate": g(d, ff), "up": g(d, ff), "down": g(ff, d),
+                            "norm1": (1 + 0.1 * r.standard_normal(d)).astype(np.float32),
+                            "norm2": (1 + 0.1 * r.standard_normal(d)).astype(np.float32)})
+    m = hip.LlamaModel(V, d, L, H, ff, eps=1e-5, rope_theta=1e4, num_kv_heads=KV)
+    m.set_embedding(w["embed"]); m.set_final_norm(w["final_norm"]); m.set_lm_head(w["lm_head"])
+    for b, lw in zip(m.blocks, w["layers"]):
+        b.set_weights(lw["w_q"], lw["w_k"], lw["w_v"], lw["w_o"]); b.set_norms(lw["norm1"], lw["norm2"])
+        b.set_ffn(lw["gate"], lw["up"], lw["down"])
+    om = tinyllama.OracleModel(w, orc)
+    toks = [int(t) for t in r.integers(0, V, 9)]
+    for i, t in enumerate(toks):   # token by token: every product of every run has one row
+        rm.assert_close(m.run([t]), om.run([t]), ATOL, RTOL, f"token {i}")
+    step_logits = m.logits()
+    m.clear_cache()
+    rm.assert_close(m.run(toks), step_logits, ATOL, RTOL, "one prompt against token by token")
+    # other weights in block 1 and another lm_head: the transposed copies are made again
+    lw = w["layers"][1]
+    lw["w_o"], lw["gate"], lw["down"] = g(H * hd, d), g(d, ff), g(ff, d)
+    m.blocks[1].set_weights(lw["w_q"], lw["w_k"], lw["w_v"], lw["w_o"]); m.blocks[1].set_ffn(lw["gate"], lw["up"], lw["down"])
+    w["lm_head"] = g(d, V)
+    m.set_lm_head(w["lm_head"])
+    om = tinyllama.OracleModel(w, orc)
+    m.clear_cache()
+    for i, t in enumerate(toks[:3]):
+        rm.assert_close(m.run([t]), om.run([t]), ATOL, RTOL, f"new weights, token {i}")
+    m.close()
+
+
 # ---- the sampler on the device ---------------------------------------------------------------
 @pytest.fixture(scope="module")
 def sampler_model(hip):
