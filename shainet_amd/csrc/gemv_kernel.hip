@@ -356,97 +356,153 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 // ---- one row of x against weights kept transposed: wt [N, K] (row n = column n of W) --------
 // Every output element is one contiguous row of wt, so a wavefront owns whole outputs: it reads
 // a row with KV4 16-byte loads per lane, all in flight at once, multiplies by the x values it
-// keeps in registers and adds up across its lanes.  Nothing crosses wavefronts: no partial sums
-// in memory, no flag words, no wait, no LDS, and a launch ends when its rows have streamed (a
-// 2048 x 2048 product: 4.8 us back to back against 8.8 us for the split product above).  What it
-// costs is the second copy of the matrix.  NACC = 2: the SwiGLU epilogue; the wavefront reads row
-// n (gate) and row N + n (up).  K = 256 KV4.  The RMSNorm prologue is done by every wavefront for
-// itself from the x values it holds (fp64 as rms_norm.cr:18-37; another order of the additions
-// than the split product's).
-// SP = 2: two wavefronts share an output, half a row each (K = 512 KV4), and add up through LDS:
-// rows of 8192 values, which one wavefront could only hold with a single wavefront per SIMD
-// (no norm prologue then, and NACC = 1).
-template <int KV4, int NACC, int SP>
+// holds and adds up across its lanes.  Nothing crosses workgroups: no partial sums in memory, no
+// flag words, no wait, and a launch ends when its rows have streamed (a 2048 x 2048 product:
+// 4.8 us back to back against 8.8 us for the split product above).  What it costs is the second
+// copy of the matrix.  NACC = 2: the SwiGLU epilogue; the wavefront reads row n (gate) and row
+// N + n (up).  SP = 2: two wavefronts share an output, half a row each, and add up through LDS
+// (rows of 8192 values; NACC = 1, no norm).  K = 256 KV4 SP.  The RMSNorm prologue is done by every
+// wavefront for itself (fp64 as rms_norm.cr:18-37; x / rms as x * (1 / rms): a division per element
+// in every wavefront cost 5 of the 26 us of a 2048 -> 2 x 8192 product), once for the
+// a.rows_per_wave consecutive outputs it takes (more than one where N is large, so that the
+// prologue does not outweigh the rows: 128 256 outputs with a wavefront each took 199 us, the
+// split product 169 us).  The next row's loads are issued before the current row is added up.
+// MULTI: a wavefront takes more than one output; only then are there registers for a second row.
+template <int KV4, int NACC, int SP, bool MULTI>
 __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
+  // x: up to 2048 values stay in registers.  Longer (half) rows: a wavefront with one output reads
+  // them again from memory (the L2), eight 16-byte pieces at a time, where they are used; one with
+  // several outputs keeps its own normed copy in LDS
+  constexpr bool XREG = KV4 <= 8, XLDS = !XREG && MULTI;
+  __shared__ __align__(16) float xs[XLDS ? 4 * 256 * KV4 : 4];
   __shared__ float half_s[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = blockIdx.x * (4 / SP) + wave / SP;  // the output this wavefront owns (or shares)
+  const int rpw = a.rows_per_wave;
+  const int n0 = (blockIdx.x * (4 / SP) + wave / SP) * rpw;  // this wavefront's first output
   const int seg = wave % SP;
   const int N = a.N;
-  constexpr int K = 256 * KV4 * SP;
-  // (with SP = 2, N is even: launch_gemvt sees to it, so both wavefronts of a pair are in or out)
-  if (n >= N) return;
-  f32x4 w[NACC][KV4];
+  constexpr int KW = 256 * KV4;  // values per wavefront and row
+  constexpr int K = KW * SP;
+  // (with SP = 2 both wavefronts of a pair see the same n0: they leave together)
+  if (n0 >= N) return;
+  auto load_row = [&](f32x4 (&w)[NACC][KV4], int n) {
 #pragma unroll
-  for (int c = 0; c < NACC; ++c) {
-    const float *row = a.w + ((long long)c * N + n) * K + seg * (256 * KV4) + 4 * lane;
+    for (int c = 0; c < NACC; ++c) {
+      const float *row = a.w + ((long long)c * N + n) * K + seg * KW + 4 * lane;
 #pragma unroll
-    for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
-  }
-  // x: up to 2048 values stay in registers; longer rows are read again, eight 16-byte pieces at
-  // a time (from the L2), where they are used, the registers being needed for the row of wt
+      for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
+    }
+  };
+  f32x4 wa[NACC][KV4], wb[MULTI ? NACC : 1][MULTI ? KV4 : 1];
+  load_row(wa, n0);
+
   constexpr int XC = KV4 < 8 ? KV4 : 8;
-  const float *xp = a.x + seg * (256 * KV4) + 4 * lane;
+  const float *xp = a.x + seg * KW + 4 * lane;
+  float *my_xs = xs + (XLDS ? wave * KW : 0) + 4 * lane;
   double rms = 1.0;  // 1 / the root mean square
   if (a.norm) {
     double sq = 0.0;
 #pragma unroll
     for (int c0 = 0; c0 < KV4; c0 += XC) {
-      f32x4 xv[XC];
+      f32x4 t[XC];
 #pragma unroll
-      for (int i = 0; i < XC; ++i) xv[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
+      for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
 #pragma unroll
       for (int i = 0; i < XC; ++i) {
-        sq += (double)xv[i].x * (double)xv[i].x + (double)xv[i].y * (double)xv[i].y;
-        sq += (double)xv[i].z * (double)xv[i].z + (double)xv[i].w * (double)xv[i].w;
+        sq += (double)t[i].x * (double)t[i].x + (double)t[i].y * (double)t[i].y;
+        sq += (double)t[i].z * (double)t[i].z + (double)t[i].w * (double)t[i].w;
       }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
-    // (x / rms as x * (1 / rms): every wavefront norms the whole row for itself, and a division
-    // per element, eight wavefronts' worth per SIMD, cost 5 of the 26 us of a 2048 -> 2 x 8192 product)
     rms = 1.0 / sqrt(sq / (double)K + a.eps);
   }
-  f32x4 acc[NACC];
+  // pieces c0 .. c0 + XC - 1 of x, normed if asked
+  auto x_pieces = [&](f32x4 (&t)[XC], int c0) {
 #pragma unroll
-  for (int c = 0; c < NACC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int c0 = 0; c0 < KV4; c0 += XC) {
-    f32x4 xv[XC];
-#pragma unroll
-    for (int i = 0; i < XC; ++i) xv[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
+    for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
     if (a.norm) {
 #pragma unroll
       for (int i = 0; i < XC; ++i) {
         f32x4 g = {1.f, 1.f, 1.f, 1.f};
-        if (a.gamma) g = *(const f32x4 *)(a.gamma + 4 * lane + 256 * (c0 + i));
-        xv[i] = f32x4{(float)(((double)xv[i].x * rms) * (double)g.x), (float)(((double)xv[i].y * rms) * (double)g.y),
-                      (float)(((double)xv[i].z * rms) * (double)g.z), (float)(((double)xv[i].w * rms) * (double)g.w)};
+        if (a.gamma) g = *(const f32x4 *)(a.gamma + seg * KW + 4 * lane + 256 * (c0 + i));
+        t[i] = f32x4{(float)(((double)t[i].x * rms) * (double)g.x), (float)(((double)t[i].y * rms) * (double)g.y),
+                     (float)(((double)t[i].z * rms) * (double)g.z), (float)(((double)t[i].w * rms) * (double)g.w)};
       }
     }
+  };
+  f32x4 xv[XREG ? KV4 : 1];
+  if constexpr (XREG || XLDS) {
 #pragma unroll
-    for (int c = 0; c < NACC; ++c)
+    for (int c0 = 0; c0 < KV4; c0 += XC) {
+      f32x4 t[XC];
+      x_pieces(t, c0);
 #pragma unroll
-      for (int i = 0; i < XC; ++i) acc[c] += w[c][c0 + i] * xv[i];
+      for (int i = 0; i < XC; ++i) {
+        if constexpr (XREG)
+          xv[c0 + i] = t[i];
+        else
+          *(f32x4 *)(my_xs + 256 * (c0 + i)) = t[i];  // read back by this lane only: no barrier
+      }
+    }
   }
-  float s[NACC];
+
+  auto finish_row = [&](const f32x4 (&w)[NACC][KV4], int n) {
+    f32x4 acc[NACC];
 #pragma unroll
-  for (int c = 0; c < NACC; ++c) {
-    s[c] = (acc[c].x + acc[c].y) + (acc[c].z + acc[c].w);
+    for (int c = 0; c < NACC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) s[c] += __shfl_xor(s[c], o);
-  }
-  if constexpr (SP == 2) {
-    if (lane == 0) half_s[wave] = s[0];
-    __syncthreads();
-    if (seg) return;
-    s[0] = half_s[wave] + half_s[wave + 1];
-  }
-  if (lane == 0) {
-    float v = s[0];
-    if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
-    if (a.epilogue == kGemvResidual) v = (float)((double)a.res[n] + (double)s[0]);
-    a.y[n] = v;
+    for (int c0 = 0; c0 < KV4; c0 += XC) {
+      f32x4 t[XC];
+      if constexpr (XREG) {
+#pragma unroll
+        for (int i = 0; i < XC; ++i) t[i] = xv[c0 + i];
+      } else if constexpr (XLDS) {
+#pragma unroll
+        for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(my_xs + 256 * (c0 + i));
+      } else {
+        x_pieces(t, c0);
+      }
+#pragma unroll
+      for (int c = 0; c < NACC; ++c)
+#pragma unroll
+        for (int i = 0; i < XC; ++i) acc[c] += w[c][c0 + i] * t[i];
+    }
+    float s[NACC];
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) {
+      s[c] = (acc[c].x + acc[c].y) + (acc[c].z + acc[c].w);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) s[c] += __shfl_xor(s[c], o);
+    }
+    if constexpr (SP == 2) {
+      __syncthreads();  // (the pair's sums of the row before have been read)
+      if (lane == 0) half_s[wave] = s[0];
+      __syncthreads();
+      s[0] = half_s[wave & ~1] + half_s[wave | 1];
+      if (seg) return;
+    }
+    if (lane == 0) {
+      float v = s[0];
+      if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
+      if (a.epilogue == kGemvResidual) v = (float)((double)a.res[n] + (double)s[0]);
+      a.y[n] = v;
+    }
+  };
+  // (with SP = 2 every wavefront of the workgroup makes the same number of turns: the rows of
+  // all pairs end together, launch_gemvt sees to it, so the barriers above are met by all)
+  if constexpr (MULTI) {
+    const int n_end = min(n0 + rpw, N);
+    for (int n = n0; n < n_end; n += 2) {
+      if (n + 1 < n_end) load_row(wb, n + 1);
+      finish_row(wa, n);
+      if (n + 1 < n_end) {
+        if (n + 2 < n_end) load_row(wa, n + 2);
+        finish_row(wb, n + 1);
+      }
+    }
+  } else {
+    finish_row(wa, n0);
   }
 }
 
@@ -549,22 +605,38 @@ hipError_t launch_gemvt(const GemvArgs &args, hipStream_t stream) {
   if (!gemvt_takes(a.T, a.K, a.N, a.epilogue, a.norm != 0) || !a.x || !a.w || !a.y) return hipErrorInvalidValue;
   if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
   if (((uintptr_t)a.x | (uintptr_t)a.w | (uintptr_t)a.gamma) & 15) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)((a.N + 3) / 4));
   const bool two = a.epilogue == kGemvSwiglu;
-#define SHAINET_LAUNCH_GEMVT(KV4_)                                                     \
-  do {                                                                                 \
-    if (two)                                                                           \
-      hipLaunchKernelGGL((gemvt_kernel<KV4_, 2, 1>), grid, dim3(256), 0, stream, a);   \
-    else                                                                               \
-      hipLaunchKernelGGL((gemvt_kernel<KV4_, 1, 1>), grid, dim3(256), 0, stream, a);   \
+  const int sp = a.K == 8192 ? 2 : 1;
+  // outputs per wavefront: one until the launch has some 16 000 wavefronts, then more
+  static const int wave_target = getenv("SHAINET_HIP_GEMVT_WAVES") ? atoi(getenv("SHAINET_HIP_GEMVT_WAVES")) : 16384;
+  int rpw = (int)(((long long)a.N * (two ? 2 : 1) * sp + wave_target - 1) / wave_target);
+  if (sp == 2) {
+    // all pairs of a workgroup must take the same number of rows: rpw divides N / 2 pairs' worth evenly
+    while ((a.N / 2) % rpw) --rpw;
+  }
+  a.rows_per_wave = rpw;
+  const int per_wg = (4 / sp) * rpw;
+  const dim3 grid((unsigned)((a.N + per_wg - 1) / per_wg));
+#define SHAINET_LAUNCH_GEMVT(KV4_)                                                            \
+  do {                                                                                        \
+    if (two && rpw > 1)                                                                       \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 2, 1, true>), grid, dim3(256), 0, stream, a);    \
+    else if (two)                                                                             \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 2, 1, false>), grid, dim3(256), 0, stream, a);   \
+    else if (rpw > 1)                                                                         \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 1, 1, true>), grid, dim3(256), 0, stream, a);    \
+    else                                                                                      \
+      hipLaunchKernelGGL((gemvt_kernel<KV4_, 1, 1, false>), grid, dim3(256), 0, stream, a);   \
   } while (0)
   switch (a.K) {
     case 1024: SHAINET_LAUNCH_GEMVT(4); break;
     case 2048: SHAINET_LAUNCH_GEMVT(8); break;
     case 4096: SHAINET_LAUNCH_GEMVT(16); break;
     default:  // 8192: two wavefronts per output
-      if (two || a.norm || (a.N & 1)) return hipErrorInvalidValue;
-      hipLaunchKernelGGL((gemvt_kernel<16, 1, 2>), dim3((unsigned)(a.N / 2)), dim3(256), 0, stream, a);
+      if (rpw > 1)
+        hipLaunchKernelGGL((gemvt_kernel<16, 1, 2, true>), grid, dim3(256), 0, stream, a);
+      else
+        hipLaunchKernelGGL((gemvt_kernel<16, 1, 2, false>), grid, dim3(256), 0, stream, a);
       break;
   }
 #undef SHAINET_LAUNCH_GEMVT
