@@ -38,6 +38,7 @@
 #include "gemm_kernel.hpp"
 
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace shainet {
 
@@ -394,6 +395,9 @@ GemmPlan plan_gemm(int T, int K, int N, long long x_stride) {
     // more pieces per tile: as many as fill one round, of at least 8 steps each, all equal; the
     // second kernel adds them
     int pieces = slots / tiles;
+    static const int pieces_knob = getenv("SHAINET_HIP_GEMM_PIECES") ? atoi(getenv("SHAINET_HIP_GEMM_PIECES")) : 0;
+    if (pieces > 16) pieces = 16;  // (128 rows of 8192 -> 2048: 32 pieces 56 us, 16 pieces 48.5 us)
+    if (pieces_knob > 0) pieces = pieces_knob;  // SHAINET_HIP_GEMM_PIECES: a tuning knob
     if (pieces > p.steps / 8) pieces = p.steps / 8;
     if (pieces < 1) pieces = 1;
     p.quota = (p.steps + pieces - 1) / pieces;

@@ -84,7 +84,11 @@ const float *transposed_twin(float **twin, bool *stale, const float *src, int ro
     *stale = true;
   }
   if (*stale) {
-    if (launch_transpose(src, *twin, rows, cols, stream) != hipSuccess) return nullptr;
+    // (waited for, once per set of weights: the copy may next be read on another stream)
+    if (launch_transpose(src, *twin, rows, cols, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
     *stale = false;
   }
   return *twin;
