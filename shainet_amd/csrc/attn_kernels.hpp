@@ -210,8 +210,9 @@ GemvPlan plan_gemv(int T, int K, int N, int epilogue, int head_dim = 0);
 hipError_t launch_gemv(const GemvArgs &a, const GemvPlan &p, hipStream_t stream);
 // The same product for one row of x against weights kept transposed (a.w: [N, K], or [2N, K] =
 // gate | up for kGemvSwiglu): a wavefront per output, nothing shared between wavefronts.
-// gemvt_takes: what it serves (one row; K 1024, 2048, 4096, or 8192 without norm and SwiGLU).
-bool gemvt_takes(int T, int K, int N, int epilogue, bool norm);
+// gemvt_takes: what it serves (one row; K 1024, 2048, 4096, or 8192 without norm and SwiGLU; the
+// kGemvQkvPrep epilogue, a.w: [(H + 2 KV) hd, K], where *prep asks for no QK-norm).
+bool gemvt_takes(int T, int K, int N, int epilogue, bool norm, const GemvPrep *prep = nullptr);
 hipError_t launch_gemvt(const GemvArgs &a, hipStream_t stream);
 
 // A pinned host int per context (block, model) that its kernels set when they give up a

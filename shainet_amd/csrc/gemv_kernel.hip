@@ -96,6 +96,34 @@ __device__ __forceinline__ void prep_tile_row(const GemvPrep &p, const float *ti
   }
 }
 
+// The same for one pair (x0 = element i, x1 = element i + hd / 2) of head row r of a single token,
+// without QK-norm (which needs the whole head): called by one lane.
+__device__ __forceinline__ void prep_pair(const GemvPrep &p, int r, int i, float x0, float x1) {
+  const int hd = p.hd, half = hd >> 1;
+  const int pos = p.start_pos;
+  const float *bias;
+  float *dst;
+  bool rotate = true;
+  if (r < p.H) {
+    bias = p.b_q ? p.b_q + r * hd : nullptr;
+    dst = p.q_rot + r * hd;
+  } else {
+    const bool is_v = r - p.H >= p.KV;
+    const int c = is_v ? r - p.H - p.KV : r - p.H;
+    bias = is_v ? (p.b_v ? p.b_v + c * hd : nullptr) : (p.b_k ? p.b_k + c * hd : nullptr);
+    dst = (is_v ? p.vc : p.kc) + ((long long)c * p.cap + pos) * hd;
+    rotate = !is_v;
+  }
+  if (bias) {
+    x0 = x0 + bias[i];
+    x1 = x1 + bias[i + half];
+  }
+  float y0 = x0, y1 = x1;
+  if (rotate) norm_rotate_pair(x0, x1, false, 1.0f, 1.0f, p.eps, hd, half, p.rope_tab[(long long)pos * half + i], y0, y1);
+  dst[i] = y0;
+  dst[i + half] = y1;
+}
+
 // NACC = 1, or 2 for the SwiGLU epilogue (gate and up accumulators).
 // PREP: the kGemvQkvPrep epilogue (NACC = 1).
 // RPI = rows of W per load instruction: 1 (a wavefront spans 256 columns) or 4
@@ -368,8 +396,13 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 // prologue does not outweigh the rows: 128 256 outputs with a wavefront each took 199 us, the
 // split product 169 us).  The next row's loads are issued before the current row is added up.
 // MULTI: a wavefront takes more than one output; only then are there registers for a second row.
-template <int KV4, int NACC, int SP, bool MULTI>
+// PREP (NACC = 2, a.N = the number of pairs): the kGemvQkvPrep epilogue of a q | k | v product without
+// QK-norm.  Output n is the pair (i, i + hd / 2) of head row r, n = r * hd / 2 + i: rows r * hd + i and
+// r * hd + i + hd / 2 of the matrix, whose two sums are all that bias, RoPE and the cache append of
+// the pair need (llama_block.cr:256-286, 332-344), so the head rows never go through memory either.
+template <int KV4, int NACC, int SP, bool MULTI, bool PREP = false>
 __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
+  static_assert(!PREP || (NACC == 2 && SP == 1 && !MULTI), "the q | k | v epilogue: one pair per wavefront");
   // x: up to 2048 values stay in registers.  Longer (half) rows: a wavefront with one output reads
   // them again from memory (the L2), eight 16-byte pieces at a time, where they are used; one with
   // several outputs keeps its own normed copy in LDS
@@ -385,10 +418,12 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   constexpr int K = KW * SP;
   // (with SP = 2 both wavefronts of a pair see the same n0: they leave together)
   if (n0 >= N) return;
+  const int half_hd = PREP ? a.prep.hd >> 1 : 1;
   auto load_row = [&](f32x4 (&w)[NACC][KV4], int n) {
 #pragma unroll
     for (int c = 0; c < NACC; ++c) {
-      const float *row = a.w + ((long long)c * N + n) * K + seg * KW + 4 * lane;
+      const long long wrow = PREP ? (long long)n + (n / half_hd + c) * half_hd : (long long)c * N + n;
+      const float *row = a.w + wrow * K + seg * KW + 4 * lane;
 #pragma unroll
       for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
     }
@@ -482,7 +517,9 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       s[0] = half_s[wave & ~1] + half_s[wave | 1];
       if (seg) return;
     }
-    if (lane == 0) {
+    if constexpr (PREP) {
+      if (lane == 0) prep_pair(a.prep, n / half_hd, n % half_hd, s[0], s[NACC - 1]);
+    } else if (lane == 0) {
       float v = s[0];
       if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
       if (a.epilogue == kGemvResidual) v = (float)((double)a.res[n] + (double)s[0]);
@@ -592,8 +629,12 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
   return hipGetLastError();
 }
 
-bool gemvt_takes(int T, int K, int N, int epilogue, bool norm) {
+bool gemvt_takes(int T, int K, int N, int epilogue, bool norm, const GemvPrep *prep) {
   if (T != 1 || N < 1) return false;
+  if (epilogue == kGemvQkvPrep) {
+    if (!prep || prep->q_norm || prep->k_norm || prep->hd < 2 || (prep->hd & 1)) return false;
+    return (K == 1024 || K == 2048 || K == 4096) && N == (prep->H + 2 * prep->KV) * prep->hd;
+  }
   // rows of 8192: two wavefronts per output, which leaves out the norm prologue and SwiGLU
   if (K == 8192) return !norm && !(N & 1) && (epilogue == kGemvPlain || epilogue == kGemvResidual);
   if (K != 1024 && K != 2048 && K != 4096) return false;
@@ -602,9 +643,24 @@ bool gemvt_takes(int T, int K, int N, int epilogue, bool norm) {
 
 hipError_t launch_gemvt(const GemvArgs &args, hipStream_t stream) {
   GemvArgs a = args;
-  if (!gemvt_takes(a.T, a.K, a.N, a.epilogue, a.norm != 0) || !a.x || !a.w || !a.y) return hipErrorInvalidValue;
+  const bool prep = a.epilogue == kGemvQkvPrep;
+  if (!gemvt_takes(a.T, a.K, a.N, a.epilogue, a.norm != 0, &a.prep) || !a.x || !a.w || (!a.y && !prep)) return hipErrorInvalidValue;
   if (a.epilogue == kGemvResidual && !a.res) return hipErrorInvalidValue;
   if (((uintptr_t)a.x | (uintptr_t)a.w | (uintptr_t)a.gamma) & 15) return hipErrorInvalidValue;
+  if (prep) {
+    const GemvPrep &q = a.prep;
+    if (q.H < 1 || q.KV < 1 || !q.rope_tab || !q.q_rot || !q.kc || !q.vc || q.start_pos < 0 || q.start_pos + 1 > q.cap)
+      return hipErrorInvalidValue;
+    a.N = a.N / 2;  // pairs, one wavefront each
+    a.rows_per_wave = 1;
+    const dim3 pgrid((unsigned)((a.N + 3) / 4));
+    switch (a.K) {
+      case 1024: hipLaunchKernelGGL((gemvt_kernel<4, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+      case 2048: hipLaunchKernelGGL((gemvt_kernel<8, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+      default: hipLaunchKernelGGL((gemvt_kernel<16, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+    }
+    return hipGetLastError();
+  }
   const bool two = a.epilogue == kGemvSwiglu;
   const int sp = a.K == 8192 ? 2 : 1;
   // outputs per wavefront: one until the launch has some 16 000 wavefronts, then more

@@ -41,8 +41,9 @@ struct shainet_llama_attn {
   float *w_qkv = nullptr, *w_o = nullptr;  // device, [in, out]; w_q | w_k | w_v side by side in one matrix
   // w_o once more, transposed ([d_model, q_dim]), for the product of a single row (launch_gemvt):
   // made on the device when such a call first needs it, made again after the weights change
-  float *w_o_t = nullptr;
-  bool w_o_t_stale = true;
+  // (and q | k | v, [q_dim + 2 kv_dim, d_model], for layers without QK-norm)
+  float *w_o_t = nullptr, *w_qkv_t = nullptr;
+  bool w_o_t_stale = true, w_qkv_t_stale = true;
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
   shainet_kv_cache *scratch_cache = nullptr;  // rows of a no-cache forward call; empty between calls
@@ -138,6 +139,8 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     Fused qkv = pre;
     qkv.epilogue = kGemvQkvPrep;
     qkv.prep = &where;
+    if (gemvt_takes(T, l->d_model, wide, qkv.epilogue, qkv.norm, &where))
+      qkv.w_t = transposed_twin(&l->w_qkv_t, &l->w_qkv_t_stale, l->w_qkv, l->d_model, wide, stream);
     if ((rc = l->proj.project(x, l->d_model, l->w_qkv, nullptr, T, l->d_model, wide, stream, qkv))) return rc;
     rc = shainet_attn_finish_prepared(l->ctx, cache, T, l->attn.p);  // 287-296
   } else {
@@ -196,7 +199,7 @@ int shainet_llama_attn_destroy(shainet_llama_attn *l) {
   if (!l) return SHAINET_HIP_OK;
   drop_context(l);
   l->proj.release();
-  for (float *p : {l->w_qkv, l->w_o, l->w_o_t})
+  for (float *p : {l->w_qkv, l->w_o, l->w_o_t, l->w_qkv_t})
     if (p) (void)hipFree(p);
   for (DevF *b : {&l->x, &l->qkv, &l->attn, &l->out}) b->release();
   l->x_pin.release();
@@ -240,7 +243,7 @@ int shainet_llama_attn_set_weights(shainet_llama_attn *l, const float *w_q, cons
   const int widths[3] = {l->q_dim, l->kv_dim, l->kv_dim};
   int rc = upload_side_by_side(&l->w_qkv, mats, widths, 3, l->d_model);
   if (!rc) rc = upload_floats(&l->w_o, w_o, (size_t)l->q_dim * l->d_model);
-  l->w_o_t_stale = true;
+  l->w_o_t_stale = l->w_qkv_t_stale = true;
   return rc;
 }
 
@@ -357,7 +360,7 @@ int shainet_llama_block_buffers(shainet_llama_block *b, LlamaBlockBuffers *out) 
       return fail(SHAINET_HIP_ERR_ALLOC, "hipMalloc failed");
     }
   // (whoever asks for the buffers is about to write the weights: the transposed copies are made again)
-  l->w_o_t_stale = b->gate_up_t_stale = b->down_t_stale = true;
+  l->w_o_t_stale = l->w_qkv_t_stale = b->gate_up_t_stale = b->down_t_stale = true;
   *out = LlamaBlockBuffers{l->w_qkv, l->w_o, b->gate_up, b->down, b->norm1, b->norm2,
                            b->d_model, l->q_dim, l->kv_dim, b->ff_hidden};
   return SHAINET_HIP_OK;

@@ -64,7 +64,7 @@ void DevF::release() {
   cap = 0;
 }
 
-// SHAINET_HIP_NO_TRANSPOSED_WEIGHTS: no second, transposed copy of W_o, gate | up and down (the
+// SHAINET_HIP_NO_TRANSPOSED_WEIGHTS: no second, transposed copy of q | k | v, W_o, gate | up and down (the
 // products of a single row then run as the split GEMV over the [in, out] matrices, like the rest)
 bool transposed_twins_wanted() {
   static const bool wanted = getenv("SHAINET_HIP_NO_TRANSPOSED_WEIGHTS") == nullptr;
@@ -132,7 +132,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
   const bool swiglu = f.epilogue == kGemvSwiglu;
   if (f.epilogue == kGemvQkvPrep && (!f.prep || T > 16 || (N & 3)))
     return llama_fail(SHAINET_HIP_ERR_ARGUMENT, "the fused q | k | v epilogue takes at most 16 rows");
-  if (f.w_t && gemvt_takes(T, K, N, f.epilogue, f.norm) && !(((uintptr_t)x | (uintptr_t)f.gamma) & 15)) {
+  if (f.w_t && gemvt_takes(T, K, N, f.epilogue, f.norm, f.prep) && !(((uintptr_t)x | (uintptr_t)f.gamma) & 15)) {
     GemvArgs a = {};
     a.x = x;
     a.x_stride = x_stride;
@@ -146,6 +146,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.K = K;
     a.N = N;
     a.epilogue = f.epilogue;
+    if (f.prep) a.prep = *f.prep;
     hipError_t e = launch_gemvt(a, stream);
     if (e != hipSuccess)
       return llama_fail(SHAINET_HIP_ERR_RUNTIME, std::string("gemv launch: ") + hipGetErrorString(e));

@@ -64,6 +64,9 @@ def _oracle_forward(ob, p, eps, x):
     (128, 8, 2, 64, 344, True, True, [20, 3, 1, 17, 1]),  # explicit head_dim, QK-norm, biases, ff % 8 == 0 only
     (256, 8, 8, 128, 1024, True, False, [33, 1, 1]),
     (30, 3, 1, None, 50, False, False, [4, 1]),           # widths not multiples of 4: the plain product kernel
+    # single rows of a layer without QK-norm: q | k | v over its transposed copy, a wavefront per RoPE pair
+    (1024, 16, 4, 64, 512, False, True, [5, 1, 1, 20, 1]),
+    (2048, 8, 2, 128, 256, False, False, [1, 1, 3, 1]),
 ])
 def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
     blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e6, seed=d + ff, norm=norm, bias=bias)
@@ -456,8 +459,8 @@ def test_long_generation_across_cache_growth_equals_one_prefill(hip):
 
 @pytest.mark.parametrize("tied", [True, False])
 def test_single_row_products_over_transposed_weights(hip, tied):
-    """One-token runs of a model whose shapes the transposed-weight product serves (W_o and gate | up
-    with K = 1024, down with K = 4096, lm_head with K = 1024): a wavefront per output over second,
+    """One-token runs of a model whose shapes the transposed-weight product serves (q | k | v, W_o and
+    gate | up with K = 1024, down with K = 4096, lm_head with K = 1024): a wavefront per output over second,
     transposed copies of the matrices, made on the device at the first such run; lm_head's is the
     embedding table itself when the two are tied (compared on the device), a copy otherwise.
     Against the oracle, and against the same tokens run as one prompt (MFMA products, no such copies);
@@ -490,7 +493,7 @@ def test_single_row_products_over_transposed_weights(hip, tied):
     rm.assert_close(m.run(toks), step_logits, ATOL, RTOL, "one prompt against token by token")
     # other weights in block 1 and another lm_head: the transposed copies are made again
     lw = w["layers"][1]
-    lw["w_o"], lw["gate"], lw["down"] = g(H * hd, d), g(d, ff), g(ff, d)
+    lw["w_q"], lw["w_v"], lw["w_o"], lw["gate"], lw["down"] = g(d, H * hd), g(d, KV * hd), g(H * hd, d), g(d, ff), g(ff, d)
     m.blocks[1].set_weights(lw["w_q"], lw["w_k"], lw["w_v"], lw["w_o"]); m.blocks[1].set_ffn(lw["gate"], lw["up"], lw["down"])
     w["lm_head"] = g(d, V)
     m.set_lm_head(w["lm_head"])
