@@ -67,6 +67,7 @@ def _oracle_forward(ob, p, eps, x):
     # single rows of a layer without QK-norm: q | k | v over its transposed copy, a wavefront per RoPE pair
     (1024, 16, 4, 64, 512, False, True, [5, 1, 1, 20, 1]),
     (2048, 8, 2, 128, 256, False, False, [1, 1, 3, 1]),
+    (4096, 8, 2, 64, 128, False, True, [1, 1, 2, 1]),
 ])
 def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
     blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e6, seed=d + ff, norm=norm, bias=bias)
@@ -457,16 +458,19 @@ def test_long_generation_across_cache_growth_equals_one_prefill(hip):
     np.testing.assert_array_equal(m.logits(), last)
 
 
-@pytest.mark.parametrize("tied", [True, False])
-def test_single_row_products_over_transposed_weights(hip, tied):
+@pytest.mark.parametrize("tied,d,H,KV,ff", [(True, 1024, 8, 2, 4096), (False, 1024, 8, 2, 4096),
+                                            # rows of 8192 in the down product: two wavefronts per output
+                                            (False, 2048, 16, 4, 8192)])
+def test_single_row_products_over_transposed_weights(hip, tied, d, H, KV, ff):
     """One-token runs of a model whose shapes the transposed-weight product serves (q | k | v, W_o and
     gate | up with K = 1024, down with K = 4096, lm_head with K = 1024): a wavefront per output over second,
     transposed copies of the matrices, made on the device at the first such run; lm_head's is the
     embedding table itself when the two are tied (compared on the device), a copy otherwise.
-    Against the oracle, and against the same tokens run as one prompt (MFMA products, no such copies);
+    (With SHAINET_HIP_GEMVT_WAVES set low, as one of the tuning-variable runs does, every wavefront
+    takes several outputs, as for a vocabulary of 128 256.)  Against the oracle, and against the same tokens run as one prompt (MFMA products, no such copies);
     then new weights in one block: the copies must follow."""
     r = np.random.default_rng(5)
-    V, d, L, H, KV, ff = 700, 1024, 2, 8, 2, 4096
+    V, L = 700, 2
     hd = d // H
     cfg = {"vocab_size": V, "hidden_size": d, "num_hidden_layers": L, "num_attention_heads": H, "num_key_value_heads": KV,
            "intermediate_size": ff, "rms_norm_eps": 1e-5, "rope_theta": 1e4}
