@@ -128,6 +128,12 @@ struct DecodeArgs {
   // instead of part_flag, and waiting ends after spin_limit polls; null / 0 otherwise
   unsigned *flag_set;
   int spin_limit;
+  // Rows of another kernel's weights to read into the L2s meanwhile (null: none): extra workgroups
+  // behind the attention's own read what the first ahead_wgs workgroups of the product
+  // gemvt_kernel<K / 256, 2, 1, false> over ahead_w ([2 ahead_n, ahead_k]) will read, from the
+  // same indices modulo 8 and so on the same XCDs.  Host-planned launches of head_dim 64 or 128 only.
+  const float *ahead_w = nullptr;
+  int ahead_k = 0, ahead_n = 0, ahead_wgs = 0;
 };
 // dev != nullptr: st gives the number of sequences only, p the grid (kDevicePlanWorkgroups), the
 // slots and the columns; everything that depends on the cached lengths is read from *dev.

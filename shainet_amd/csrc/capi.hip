@@ -140,6 +140,9 @@ struct shainet_attn_ctx {
   float *d_bq = nullptr, *d_bk = nullptr, *d_bv = nullptr;
   float2 *d_rope = nullptr;
   int rope_positions = 0;
+  // DecodeArgs::ahead_* of the next decode launch (shainet_attn_read_ahead); forgotten after it
+  const float *ahead_w = nullptr;
+  int ahead_k = 0, ahead_n = 0, ahead_wgs = 0;
   hipStream_t stream = nullptr;      // where work is issued
   hipStream_t own_stream = nullptr;  // created with the context, destroyed with it
   DevBuf q_rot, partials, in_q, in_k, in_v, out;
@@ -348,6 +351,13 @@ int run_attention(shainet_attn_ctx *c, const float *q_rot, float *kc, float *vc,
     d.out = out;
     d.error = c->error;
     d.spin_limit = c->test_lose_marks ? 2000 : 0;
+    if (!ws) {  // (asked for by the caller of this one launch)
+      d.ahead_w = c->ahead_w;
+      d.ahead_k = c->ahead_k;
+      d.ahead_n = c->ahead_n;
+      d.ahead_wgs = c->ahead_wgs;
+    }
+    c->ahead_w = nullptr;
     if (prep) {
       e = launch_prep(*prep, st, sh, total_tokens, stream);
       if (e != hipSuccess) return hip_fail(e, "prep launch");
@@ -1080,6 +1090,14 @@ int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int n
 void shainet_attn_commit_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens) {
   kc->len[0] += new_tokens;
   c->last_rows = 0;
+}
+
+void shainet_attn_read_ahead(shainet_attn_ctx *c, const float *w, int k, int n, int wgs) {
+  if (!c) return;
+  c->ahead_w = w;
+  c->ahead_k = k;
+  c->ahead_n = n;
+  c->ahead_wgs = wgs;
 }
 
 int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out) {

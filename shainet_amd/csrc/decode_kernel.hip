@@ -185,12 +185,38 @@ constexpr int kFlagSpinLimit = 1 << 21;  // polls of about a microsecond each: s
 // same as part_flag except in the test of that give-up, which sends them elsewhere.
 // DEV: the sequence table and the spans come from *dev (device memory, written by
 // decode_plan_kernel earlier on the stream) instead of from the kernel arguments.
-template <int HD, int NW, bool DEV, bool PAD>
+struct ReadAhead {
+  const float *w;  // [2 n, k]
+  int k, n, first_wg;
+};
+// AHEAD: workgroups from ah.first_wg on (a multiple of 8) do not attend: workgroup first_wg + j
+// reads the rows 4 j .. 4 j + 3 and n + the same of ah.w with ordinary loads and drops them, so
+// that the launch that needs them next finds them in its XCD's L2 (a decode step of one sequence
+// leaves the memory system idle while it waits on its chain of dependent loads).
+template <int HD, int NW, bool DEV, bool PAD, bool AHEAD = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 && HD <= 128 ? 2 : 1) void decode_splitk_kernel(
     const float *__restrict__ q_rot, const float *__restrict__ kc, const float *__restrict__ vc,
     float *__restrict__ out, float *part_o, float *part_ml, unsigned *part_flag, unsigned *flag_set,
     int spin_limit, int *error, SeqTable st_arg, Shape sh, int tiles_per_wg_arg, SpanTable sp_arg, int total_tiles_arg,
-    int n_slots, int pstride, float c, unsigned rotate, const DecodeDevicePlan *__restrict__ dev) {
+    int n_slots, int pstride, float c, unsigned rotate, const DecodeDevicePlan *__restrict__ dev, ReadAhead ah) {
+  if constexpr (AHEAD) {
+    if ((int)blockIdx.x >= ah.first_wg) {
+      const int row = 4 * ((int)blockIdx.x - ah.first_wg) + (int)(threadIdx.x >> 6);
+      if (row >= ah.n) return;
+      const int pieces = ah.k >> 8;  // 16-byte pieces per lane and row
+      for (int half = 0; half < 2; ++half) {
+        const float *p = ah.w + ((long long)half * ah.n + row) * ah.k + 4 * (threadIdx.x & 63);
+        for (int i0 = 0; i0 < pieces; i0 += 8) {
+          f32x4 v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = *(const f32x4 *)(p + 256 * min(i0 + u, pieces - 1));
+#pragma unroll
+          for (int u = 0; u < 8; ++u) asm volatile("" : : "v"(v[u]));
+        }
+      }
+      return;
+    }
+  }
   using C = DecodeCfg<HD>;
   const SeqTable &st = DEV ? dev->st : st_arg;
   const SpanTable &sp = DEV ? dev->spans : sp_arg;
@@ -692,6 +718,16 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
   // before / after (nullable) receive the kernel's own first and last clock reading, not the
   // time at which the stream reached them: what is between two kernels stays out
   dim3 grid((unsigned)p.n_wgs), block(64 * kDecodeWaves);
+  ReadAhead ah = {nullptr, 0, 0, 0};
+  if (d.ahead_w && d.ahead_wgs > 0 && !dev && !before && !after && (sh.hd == 64 || sh.hd == 128) && d.ahead_k >= 256 &&
+      (d.ahead_k & 255) == 0 && d.ahead_n > 0) {
+    ah.w = d.ahead_w;
+    ah.k = d.ahead_k;
+    ah.n = d.ahead_n;
+    ah.first_wg = (p.n_wgs + 7) / 8 * 8;
+    const int most = (d.ahead_n + 3) / 4;
+    grid.x = (unsigned)(ah.first_wg + (d.ahead_wgs < most ? d.ahead_wgs : most));
+  }
   // SHAINET_HIP_DECODE_NO_ROTATE: every workgroup walks its segments from their first tile (for
   // comparison); SHAINET_HIP_DECODE_ROTATE=n: starts spread over the first n tiles only
   static const unsigned rotate = getenv("SHAINET_HIP_DECODE_NO_ROTATE") ? 0u
@@ -701,7 +737,7 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
 #define SHAINET_DECODE_LAUNCH(HD_, DEV_, PAD_)                                                                      \
   SHAINET_LAUNCH_TIMED((decode_splitk_kernel<HD_, kDecodeWaves, DEV_, PAD_>), grid, block, 0, stream, before,      \
                        after, d.q_rot, d.kc, d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit,       \
-                       d.error, st, sh, p.tiles_per_wg, p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev)
+                       d.error, st, sh, p.tiles_per_wg, p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev, ah)
 #define SHAINET_DECODE_LAUNCH_HD(HD_, PAD_) \
   do {                                      \
     if (dev)                                \
@@ -709,7 +745,15 @@ hipError_t launch_decode(const DecodeArgs &d, const SeqTable &st, const Shape &s
     else                                    \
       SHAINET_DECODE_LAUNCH(HD_, false, PAD_); \
   } while (0)
-  if (sh.hd == 64)
+  if (ah.w && sh.hd == 64)
+    hipLaunchKernelGGL((decode_splitk_kernel<64, kDecodeWaves, false, false, true>), grid, block, 0, stream, d.q_rot, d.kc,
+                       d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg,
+                       p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev, ah);
+  else if (ah.w)
+    hipLaunchKernelGGL((decode_splitk_kernel<128, kDecodeWaves, false, false, true>), grid, block, 0, stream, d.q_rot, d.kc,
+                       d.vc, d.out, part_o, part_ml, d.part_flag, flag_set, spin_limit, d.error, st, sh, p.tiles_per_wg,
+                       p.spans, p.total_tiles, p.n_slots, p.cols, c, rotate, dev, ah);
+  else if (sh.hd == 64)
     SHAINET_DECODE_LAUNCH_HD(64, false);
   else if (sh.hd == 128)
     SHAINET_DECODE_LAUNCH_HD(128, false);

@@ -106,8 +106,12 @@ void set_vec(std::vector<float> &v, bool &has, const float *src, int n) {
 // no_cache: attention_full_cpu (209-243) instead: the same arithmetic from
 // position 0 over the rows of this call alone; they go through a scratch cache
 // that is empty again afterwards, and the block's own cache is not touched.
+struct AheadRows {  // the transposed gate | up weights ([2 n, k]) the block's next product but one will read
+  const float *wt;
+  int k, n;
+};
 int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out, const Fused &pre = Fused(),
-                        const float *residual = nullptr, bool no_cache = false) {
+                        const float *residual = nullptr, bool no_cache = false, const AheadRows *ahead = nullptr) {
   if (!l->w_qkv) return fail(SHAINET_HIP_ERR_ARGUMENT, "weights not set");
   int rc = ensure_context(l);
   if (rc) return rc;
@@ -142,6 +146,12 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     if (gemvt_takes(T, l->d_model, wide, qkv.epilogue, qkv.norm, &where))
       qkv.w_t = transposed_twin(&l->w_qkv_t, &l->w_qkv_t_stale, l->w_qkv, l->d_model, wide, stream);
     if ((rc = l->proj.project(x, l->d_model, l->w_qkv, nullptr, T, l->d_model, wide, stream, qkv))) return rc;
+    // One row: the attention launch leaves the memory system idle while it waits on its chain of
+    // dependent loads, and takes along workgroups that read the first rows of the gate | up
+    // weights into the L2s (8 MB: 1134 -> 1120 us per token of the 1B shape; 17 MB and more
+    // slow the attention's own chain down by more than the product gains)
+    static const int ahead_wgs = getenv("SHAINET_HIP_READ_AHEAD_WGS") ? atoi(getenv("SHAINET_HIP_READ_AHEAD_WGS")) : 128;
+    if (ahead && ahead->wt && ahead_wgs > 0 && T == 1) shainet_attn_read_ahead(l->ctx, ahead->wt, ahead->k, ahead->n, ahead_wgs);
     rc = shainet_attn_finish_prepared(l->ctx, cache, T, l->attn.p);  // 287-296
   } else {
     if ((rc = l->proj.project(x, l->d_model, l->w_qkv, l->qkv.p, T, l->d_model, wide, stream, pre))) return rc;
@@ -322,14 +332,15 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
   n1.norm = true;
   n1.gamma = b->norm1;
   n1.eps = b->eps;
-  if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x, no_cache))) return rc;
-  // hidden = silu(normed2 * gate_proj) * (normed2 * up_proj), normed2 = @norm2.forward(h)
   Fused gate;
   gate.norm = true;
   gate.gamma = b->norm2;
   gate.eps = b->eps;
   gate.epilogue = kGemvSwiglu;
   if (gemvt_takes(T, d, ff, gate.epilogue, true)) gate.w_t = transposed_twin(&b->gate_up_t, &b->gate_up_t_stale, b->gate_up, d, 2 * ff, stream);
+  const AheadRows ahead = {gate.w_t, d, ff};
+  if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x, no_cache, &ahead))) return rc;
+  // hidden = silu(normed2 * gate_proj) * (normed2 * up_proj), normed2 = @norm2.forward(h)
   if ((rc = l->proj.project(b->h.p, d, b->gate_up, b->hidden.p, T, d, ff, stream, gate))) return rc;
   // out = h + hidden * down_proj
   Fused down;

@@ -22,6 +22,10 @@ struct GemvPrep;
 }
 int shainet_attn_begin_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, shainet::GemvPrep *where);
 int shainet_attn_finish_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens, float *out);
+// capi.hip: the next decode launch of the context (finish_prepared for a few rows) also reads, in
+// workgroups of its own, what the first `wgs` workgroups of the one-row SwiGLU product over the
+// transposed weights w ([2 n, k]) will read, into the L2s (DecodeArgs::ahead_w)
+void shainet_attn_read_ahead(shainet_attn_ctx *c, const float *w, int k, int n, int wgs);
 // capi.hip: instead of finish, when the caller's own kernel appended the rows and attended over them
 void shainet_attn_commit_prepared(shainet_attn_ctx *c, shainet_kv_cache *kc, int new_tokens);
 // capi.hip: the pinned host word a context's kernels report a given-up wait into; a block or a

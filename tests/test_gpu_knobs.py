@@ -26,7 +26,8 @@ SETTINGS = [
     {"SHAINET_HIP_PREFILL_GROUPS": "2", "SHAINET_HIP_PREFILL_WGS_PER_CU": "2"},
     {"SHAINET_HIP_NO_FUSED_PREP": "1"},                         # q | k | v product without the prep epilogue
     {"SHAINET_HIP_NO_TRANSPOSED_WEIGHTS": "1"},                 # one-row products over the [in, out] matrices only
-    {"SHAINET_HIP_GEMVT_WAVES": "300"},                         # ... over the transposed ones, several outputs per wavefront
+    # ... over the transposed ones, several outputs per wavefront; more rows read ahead beside the attention
+    {"SHAINET_HIP_GEMVT_WAVES": "300", "SHAINET_HIP_READ_AHEAD_WGS": "700"},
 ]
 
 
