@@ -414,7 +414,7 @@ def model_decode(sa, np, steps, ctx_len=512):
 
 # The kernels the two roofline objects of the bench line price, and the workloads they are priced on.
 ROOFLINE_KERNELS = {
-    "roofline": ("decode_splitk_kernel<128, 4, false, false>", "qwen3_8b_decode_b16_ctx2048-8192"),
+    "roofline": ("decode_splitk_kernel<128, 4, false, false, false>", "qwen3_8b_decode_b16_ctx2048-8192"),
     "roofline_prefill": ("prefill_turns_kernel<64, 2, false>", "llama1b_prefill_t2048"),
 }
 
