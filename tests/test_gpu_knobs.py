@@ -29,6 +29,8 @@ SETTINGS = [
     # ... over the transposed ones, several outputs per wavefront; more rows read ahead beside the attention
     {"SHAINET_HIP_GEMVT_WAVES": "300", "SHAINET_HIP_READ_AHEAD_WGS": "700"},
 ]
+# the model with rows of 8192 (its oracle takes 20 s) runs again only where the setting is about its products
+WIDE_TOO = ("SHAINET_HIP_GEMVT_WAVES",)
 
 
 @pytest.mark.parametrize("setting", SETTINGS, ids=[",".join(f"{k[12:]}={v}" for k, v in s.items()) for s in SETTINGS])
@@ -36,7 +38,8 @@ def test_parity_subset_with_tuning_variable(setting):
     env = dict(os.environ)
     env.update(setting)
     cmd = [sys.executable, "-u", "-m", "pytest", os.path.join(HERE, "test_gpu_parity.py"), os.path.join(HERE, "test_gpu_model.py"),
-           "-x", "-q", "-m", "gpu", "-k", SUBSET, "--timeout", "120", "--timeout-method", "thread", "-p", "no:cacheprovider"]
+           "-x", "-q", "-m", "gpu", "-k", SUBSET if any(k in setting for k in WIDE_TOO) else f"({SUBSET}) and not 8192",
+           "--timeout", "120", "--timeout-method", "thread", "-p", "no:cacheprovider"]
     done = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=600)
     tail = (done.stdout + done.stderr)[-3000:]
     assert done.returncode == 0, tail

@@ -64,12 +64,24 @@ def _oracle_forward(ob, p, eps, x):
     (128, 8, 2, 64, 344, True, True, [20, 3, 1, 17, 1]),  # explicit head_dim, QK-norm, biases, ff % 8 == 0 only
     (256, 8, 8, 128, 1024, True, False, [33, 1, 1]),
     (30, 3, 1, None, 50, False, False, [4, 1]),           # widths not multiples of 4: the plain product kernel
-    # single rows of a layer without QK-norm: q | k | v over its transposed copy, a wavefront per RoPE pair
-    (1024, 16, 4, 64, 512, False, True, [5, 1, 1, 20, 1]),
-    (2048, 8, 2, 128, 256, False, False, [1, 1, 3, 1]),
-    (4096, 8, 2, 64, 128, False, True, [1, 1, 2, 1]),
 ])
 def test_block_forward_cached_matches_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
+    _block_calls_match_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts)
+
+
+@pytest.mark.parametrize("d,H,KV,hd,ff,bias,Ts", [
+    (1024, 16, 4, 64, 512, True, [5, 1, 1, 20, 1]),
+    (2048, 8, 2, 128, 256, False, [1, 1, 3, 1]),
+    (4096, 8, 2, 64, 128, True, [1, 1, 2, 1]),
+])
+def test_block_steps_of_one_row_in_wide_layers(hip, d, H, KV, hd, ff, bias, Ts):
+    """Single rows of a layer without QK-norm whose width the one-row products over transposed
+    weights serve: q | k | v with a wavefront per RoPE pair (bias, rotation and the cache append in
+    its epilogue), rows of 1024, 2048 and 4096 values."""
+    _block_calls_match_oracle(hip, d, H, KV, hd, ff, False, bias, Ts)
+
+
+def _block_calls_match_oracle(hip, d, H, KV, hd, ff, norm, bias, Ts):
     blk, ob, p, r, eps = _block_pair(hip, d, H, KV, hd, ff, 1e6, seed=d + ff, norm=norm, bias=bias)
     for i, T in enumerate(Ts):
         x = r.standard_normal((T, d)).astype(np.float32)
