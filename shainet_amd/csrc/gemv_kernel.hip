@@ -390,8 +390,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 // copy of the matrix.  NACC = 2: the SwiGLU epilogue; the wavefront reads row n (gate) and row
 // N + n (up).  SP = 2: two wavefronts share an output, half a row each, and add up through LDS
 // (rows of 8192 values; NACC = 1, no norm).  K = 256 KV4 SP.  The RMSNorm prologue is done by every
-// wavefront for itself (fp64 as rms_norm.cr:18-37; x / rms as x * (1 / rms): a division per element
-// in every wavefront cost 5 of the 26 us of a 2048 -> 2 x 8192 product), once for the
+// wavefront for itself: the mean of squares in fp64 as rms_norm.cr:18-37, and the factor 1 / rms
+// applied to the finished sum, sum_k w[n][k] (x[k] gamma[k]), rather than to every x[k] (a division per
+// element in every wavefront cost 5 of the 26 us of a 2048 -> 2 x 8192 product, and two fp64
+// products per element, on the path between x and the first multiply-add, still 1.4 us), once for the
 // a.rows_per_wave consecutive outputs it takes (more than one where N is large, so that the
 // prologue does not outweigh the rows: 128 256 outputs with a wavefront each took 199 us, the
 // split product 169 us).  The next row's loads are issued before the current row is added up.
@@ -461,8 +463,7 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       for (int i = 0; i < XC; ++i) {
         f32x4 g = {1.f, 1.f, 1.f, 1.f};
         if (a.gamma) g = *(const f32x4 *)(a.gamma + seg * KW + 4 * lane + 256 * (c0 + i));
-        t[i] = f32x4{(float)(((double)t[i].x * rms) * (double)g.x), (float)(((double)t[i].y * rms) * (double)g.y),
-                     (float)(((double)t[i].z * rms) * (double)g.z), (float)(((double)t[i].w * rms) * (double)g.w)};
+        t[i] = t[i] * g;  // (1 / rms multiplies the finished sum instead of every element)
       }
     }
   };
@@ -516,6 +517,10 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       __syncthreads();
       s[0] = half_s[wave & ~1] + half_s[wave | 1];
       if (seg) return;
+    }
+    if (a.norm) {
+#pragma unroll
+      for (int c = 0; c < NACC; ++c) s[c] = (float)((double)s[c] * rms);
     }
     if constexpr (PREP) {
       if (lane == 0) prep_pair(a.prep, n / half_hd, n % half_hd, s[0], s[NACC - 1]);
