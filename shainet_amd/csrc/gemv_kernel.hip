@@ -398,13 +398,15 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvArgs a) {
 // prologue does not outweigh the rows: 128 256 outputs with a wavefront each took 199 us, the
 // split product 169 us).  The next row's loads are issued before the current row is added up.
 // MULTI: a wavefront takes more than one output; only then are there registers for a second row.
-// PREP (NACC = 2, a.N = the number of pairs): the kGemvQkvPrep epilogue of a q | k | v product without
+// PREP (NACC = 1, a.N = the number of pairs): the kGemvQkvPrep epilogue of a q | k | v product without
 // QK-norm.  Output n is the pair (i, i + hd / 2) of head row r, n = r * hd / 2 + i: rows r * hd + i and
 // r * hd + i + hd / 2 of the matrix, whose two sums are all that bias, RoPE and the cache append of
 // the pair need (llama_block.cr:256-286, 332-344), so the head rows never go through memory either.
+// A workgroup takes two pairs: wavefronts 0 and 1 their lower rows, 2 and 3 their upper rows, and
+// the sums meet in LDS (a wavefront per pair, two rows each, took 0.85 us longer for 3072 rows).
 template <int KV4, int NACC, int SP, bool MULTI, bool PREP = false>
 __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
-  static_assert(!PREP || (NACC == 2 && SP == 1 && !MULTI), "the q | k | v epilogue: one pair per wavefront");
+  static_assert(!PREP || (NACC == 1 && SP == 1 && !MULTI), "the q | k | v epilogue: one row per wavefront");
   // x: up to 2048 values stay in registers.  Longer (half) rows: a wavefront with one output reads
   // them again from memory (the L2), eight 16-byte pieces at a time, where they are used; one with
   // several outputs keeps its own normed copy in LDS
@@ -413,18 +415,23 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   __shared__ float half_s[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rpw = a.rows_per_wave;
-  const int n0 = (blockIdx.x * (4 / SP) + wave / SP) * rpw;  // this wavefront's first output
-  const int seg = wave % SP;
   const int N = a.N;
+  const int n_own = PREP ? blockIdx.x * 2 + (wave & 1) : (blockIdx.x * (4 / SP) + wave / SP) * rpw;
+  // (PREP: an odd number of pairs leaves two wavefronts of the last workgroup without one: they go
+  // through the motions on the last pair, for the barrier's sake, and store nothing)
+  const bool live = n_own < N;
+  const int n0 = PREP ? min(n_own, N - 1) : n_own;  // this wavefront's first output
+  const int seg = wave % SP;
   constexpr int KW = 256 * KV4;  // values per wavefront and row
   constexpr int K = KW * SP;
   // (with SP = 2 both wavefronts of a pair see the same n0: they leave together)
-  if (n0 >= N) return;
+  if (!PREP && !live) return;
   const int half_hd = PREP ? a.prep.hd >> 1 : 1;
+  const int upper = PREP ? wave >> 1 : 0;
   auto load_row = [&](f32x4 (&w)[NACC][KV4], int n) {
 #pragma unroll
     for (int c = 0; c < NACC; ++c) {
-      const long long wrow = PREP ? (long long)n + (n / half_hd + c) * half_hd : (long long)c * N + n;
+      const long long wrow = PREP ? (long long)n + (n / half_hd + upper) * half_hd : (long long)c * N + n;
       const float *row = a.w + wrow * K + seg * KW + 4 * lane;
 #pragma unroll
       for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
@@ -523,7 +530,9 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       for (int c = 0; c < NACC; ++c) s[c] = (float)((double)s[c] * rms);
     }
     if constexpr (PREP) {
-      if (lane == 0) prep_pair(a.prep, n / half_hd, n % half_hd, s[0], s[NACC - 1]);
+      if (lane == 0) half_s[wave] = s[0];
+      __syncthreads();
+      if (wave < 2 && lane == 0 && live) prep_pair(a.prep, n / half_hd, n % half_hd, half_s[wave], half_s[wave + 2]);
     } else if (lane == 0) {
       float v = s[0];
       if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
@@ -656,13 +665,13 @@ hipError_t launch_gemvt(const GemvArgs &args, hipStream_t stream) {
     const GemvPrep &q = a.prep;
     if (q.H < 1 || q.KV < 1 || !q.rope_tab || !q.q_rot || !q.kc || !q.vc || q.start_pos < 0 || q.start_pos + 1 > q.cap)
       return hipErrorInvalidValue;
-    a.N = a.N / 2;  // pairs, one wavefront each
+    a.N = a.N / 2;  // pairs, two per workgroup
     a.rows_per_wave = 1;
-    const dim3 pgrid((unsigned)((a.N + 3) / 4));
+    const dim3 pgrid((unsigned)((a.N + 1) / 2));
     switch (a.K) {
-      case 1024: hipLaunchKernelGGL((gemvt_kernel<4, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
-      case 2048: hipLaunchKernelGGL((gemvt_kernel<8, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
-      default: hipLaunchKernelGGL((gemvt_kernel<16, 2, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+      case 1024: hipLaunchKernelGGL((gemvt_kernel<4, 1, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+      case 2048: hipLaunchKernelGGL((gemvt_kernel<8, 1, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
+      default: hipLaunchKernelGGL((gemvt_kernel<16, 1, 1, false, true>), pgrid, dim3(256), 0, stream, a); break;
     }
     return hipGetLastError();
   }
