@@ -97,31 +97,48 @@ __device__ __forceinline__ void prep_tile_row(const GemvPrep &p, const float *ti
 }
 
 // The same for one pair (x0 = element i, x1 = element i + hd / 2) of head row r of a single token,
-// without QK-norm (which needs the whole head): called by one lane.
-__device__ __forceinline__ void prep_pair(const GemvPrep &p, int r, int i, float x0, float x1) {
+// without QK-norm (which needs the whole head), in two steps: what does not depend on the sums (where
+// the pair goes, its bias values, its cos and sin) is asked for while the weights are still on
+// their way, so that no load stands between the finished sums and the stores.
+struct PairTarget {
+  float *dst;      // element i of the head row in q_rot or in the cache
+  int half;
+  float b0, b1;    // bias of the two elements (0 without one)
+  bool has_bias, rotate;
+  float2 cs;
+};
+__device__ __forceinline__ PairTarget prep_pair_begin(const GemvPrep &p, int r, int i) {
+  PairTarget t;
   const int hd = p.hd, half = hd >> 1;
   const int pos = p.start_pos;
   const float *bias;
-  float *dst;
-  bool rotate = true;
+  t.rotate = true;
   if (r < p.H) {
     bias = p.b_q ? p.b_q + r * hd : nullptr;
-    dst = p.q_rot + r * hd;
+    t.dst = p.q_rot + r * hd + i;
   } else {
     const bool is_v = r - p.H >= p.KV;
     const int c = is_v ? r - p.H - p.KV : r - p.H;
     bias = is_v ? (p.b_v ? p.b_v + c * hd : nullptr) : (p.b_k ? p.b_k + c * hd : nullptr);
-    dst = (is_v ? p.vc : p.kc) + ((long long)c * p.cap + pos) * hd;
-    rotate = !is_v;
+    t.dst = (is_v ? p.vc : p.kc) + ((long long)c * p.cap + pos) * hd + i;
+    t.rotate = !is_v;
   }
-  if (bias) {
-    x0 = x0 + bias[i];
-    x1 = x1 + bias[i + half];
+  t.half = half;
+  t.has_bias = bias != nullptr;
+  t.b0 = bias ? bias[i] : 0.f;
+  t.b1 = bias ? bias[i + half] : 0.f;
+  t.cs = p.rope_tab[(long long)pos * half + i];
+  return t;
+}
+__device__ __forceinline__ void prep_pair_end(const GemvPrep &p, const PairTarget &t, float x0, float x1) {
+  if (t.has_bias) {
+    x0 = x0 + t.b0;
+    x1 = x1 + t.b1;
   }
   float y0 = x0, y1 = x1;
-  if (rotate) norm_rotate_pair(x0, x1, false, 1.0f, 1.0f, p.eps, hd, half, p.rope_tab[(long long)pos * half + i], y0, y1);
-  dst[i] = y0;
-  dst[i + half] = y1;
+  if (t.rotate) norm_rotate_pair(x0, x1, false, 1.0f, 1.0f, p.eps, p.hd, t.half, t.cs, y0, y1);
+  t.dst[0] = y0;
+  t.dst[t.half] = y1;
 }
 
 // NACC = 1, or 2 for the SwiGLU epilogue (gate and up accumulators).
@@ -439,6 +456,12 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   };
   f32x4 wa[NACC][KV4], wb[MULTI ? NACC : 1][MULTI ? KV4 : 1];
   load_row(wa, n0);
+  // what the epilogue of the first output reads besides: asked for now, behind the weights
+  const bool residual = !PREP && a.epilogue == kGemvResidual;
+  float res_first = 0.f;
+  if (residual) res_first = a.res[n0];
+  PairTarget target = {};
+  if constexpr (PREP) target = prep_pair_begin(a.prep, n0 / half_hd, n0 % half_hd);
 
   constexpr int XC = KV4 < 8 ? KV4 : 8;
   const float *xp = a.x + seg * KW + 4 * lane;
@@ -490,7 +513,7 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     }
   }
 
-  auto finish_row = [&](const f32x4 (&w)[NACC][KV4], int n) {
+  auto finish_row = [&](const f32x4 (&w)[NACC][KV4], int n, float res_v) {
     f32x4 acc[NACC];
 #pragma unroll
     for (int c = 0; c < NACC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -532,11 +555,11 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     if constexpr (PREP) {
       if (lane == 0) half_s[wave] = s[0];
       __syncthreads();
-      if (wave < 2 && lane == 0 && live) prep_pair(a.prep, n / half_hd, n % half_hd, half_s[wave], half_s[wave + 2]);
+      if (wave < 2 && lane == 0 && live) prep_pair_end(a.prep, target, half_s[wave], half_s[wave + 2]);
     } else if (lane == 0) {
       float v = s[0];
       if (a.epilogue == kGemvSwiglu) v = swiglu1(s[0], s[NACC - 1]);
-      if (a.epilogue == kGemvResidual) v = (float)((double)a.res[n] + (double)s[0]);
+      if (residual) v = (float)((double)res_v + (double)s[0]);
       a.y[n] = v;
     }
   };
@@ -544,16 +567,23 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   // all pairs end together, launch_gemvt sees to it, so the barriers above are met by all)
   if constexpr (MULTI) {
     const int n_end = min(n0 + rpw, N);
+    float res_a = res_first, res_b = 0.f;  // the residual values travel with the rows' loads
     for (int n = n0; n < n_end; n += 2) {
-      if (n + 1 < n_end) load_row(wb, n + 1);
-      finish_row(wa, n);
       if (n + 1 < n_end) {
-        if (n + 2 < n_end) load_row(wa, n + 2);
-        finish_row(wb, n + 1);
+        load_row(wb, n + 1);
+        if (residual) res_b = a.res[n + 1];
+      }
+      finish_row(wa, n, res_a);
+      if (n + 1 < n_end) {
+        if (n + 2 < n_end) {
+          load_row(wa, n + 2);
+          if (residual) res_a = a.res[n + 2];
+        }
+        finish_row(wb, n + 1, res_b);
       }
     }
   } else {
-    finish_row(wa, n0);
+    finish_row(wa, n0, res_first);
   }
 }
 
