@@ -707,8 +707,9 @@ hipError_t launch_gemvt(const GemvArgs &args, hipStream_t stream) {
   }
   const bool two = a.epilogue == kGemvSwiglu;
   const int sp = a.K == 8192 ? 2 : 1;
-  // outputs per wavefront: one until the launch has some 16 000 wavefronts, then more
-  static const int wave_target = getenv("SHAINET_HIP_GEMVT_WAVES") ? atoi(getenv("SHAINET_HIP_GEMVT_WAVES")) : 16384;
+  // outputs per wavefront: one until the launch has some 32 000 wavefronts, then more (128 256
+  // outputs: 4 per wavefront; 8 per wavefront were 5 us slower, 2 per wavefront 11 us)
+  static const int wave_target = getenv("SHAINET_HIP_GEMVT_WAVES") ? atoi(getenv("SHAINET_HIP_GEMVT_WAVES")) : 32768;
   int rpw = (int)(((long long)a.N * (two ? 2 : 1) * sp + wave_target - 1) / wave_target);
   if (sp == 2) {
     // all pairs of a workgroup must take the same number of rows: rpw divides N / 2 pairs' worth evenly
