@@ -289,13 +289,15 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(const float *__restrict
 }
 
 // 32 x 32 tiles through LDS: coalesced on both sides
+// (row_scale, nullable: row r of src is multiplied by row_scale[r] on its way)
 __global__ __launch_bounds__(256) void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int rows,
-                                                        int cols) {
+                                                        int cols, const float *__restrict__ row_scale) {
   __shared__ float tile[32][33];
   const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
   for (int i = ty; i < 32; i += 8)
-    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = src[(long long)(r0 + i) * cols + c0 + tx];
+    if (r0 + i < rows && c0 + tx < cols)
+      tile[i][tx] = src[(long long)(r0 + i) * cols + c0 + tx] * (row_scale ? row_scale[r0 + i] : 1.0f);
   __syncthreads();
   for (int i = ty; i < 32; i += 8)
     if (c0 + i < cols && r0 + tx < rows) dst[(long long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
@@ -324,10 +326,10 @@ hipError_t launch_transposed_differ(const float *a, const float *b, int rows, in
   return hipGetLastError();
 }
 
-hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream) {
+hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream, const float *row_scale) {
   if (!src || !dst || rows < 1 || cols < 1 || (rows + 31) / 32 > 65535) return hipErrorInvalidValue;
   hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32)), dim3(256), 0,
-                     stream, src, dst, rows, cols);
+                     stream, src, dst, rows, cols, row_scale);
   return hipGetLastError();
 }
 

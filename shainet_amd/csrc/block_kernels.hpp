@@ -11,7 +11,8 @@ namespace shainet {
 hipError_t launch_rmsnorm(const float *x, long long x_stride, const float *gamma, float *out, int rows, int cols,
                           double eps, hipStream_t stream);
 // dst[c, r] = src[r, c]: src is [rows, cols], dst [cols, rows], both dense
-hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream);
+hipError_t launch_transpose(const float *src, float *dst, int rows, int cols, hipStream_t stream,
+                            const float *row_scale = nullptr);
 // *differ (a device int the caller has set to 0) becomes 1 when a [rows, cols] is not, bit for bit,
 // the transpose of b [cols, rows]
 hipError_t launch_transposed_differ(const float *a, const float *b, int rows, int cols, int *differ, hipStream_t stream);

@@ -44,6 +44,8 @@ struct shainet_llama_attn {
   // (and q | k | v, [q_dim + 2 kv_dim, d_model], for layers without QK-norm)
   float *w_o_t = nullptr, *w_qkv_t = nullptr;
   bool w_o_t_stale = true, w_qkv_t_stale = true;
+  // the norm weights multiplied into the rows of w_qkv_t (null: none), and whether any were
+  const float *w_qkv_t_gamma = nullptr;
   shainet_attn_ctx *ctx = nullptr;
   shainet_kv_cache *cache = nullptr;
   shainet_kv_cache *scratch_cache = nullptr;  // rows of a no-cache forward call; empty between calls
@@ -143,8 +145,15 @@ int attn_forward_device(shainet_llama_attn *l, const float *x, int T, float *out
     Fused qkv = pre;
     qkv.epilogue = kGemvQkvPrep;
     qkv.prep = &where;
-    if (gemvt_takes(T, l->d_model, wide, qkv.epilogue, qkv.norm, &where))
-      qkv.w_t = transposed_twin(&l->w_qkv_t, &l->w_qkv_t_stale, l->w_qkv, l->d_model, wide, stream);
+    if (gemvt_takes(T, l->d_model, wide, qkv.epilogue, qkv.norm, &where)) {
+      // the copy carries the weights of the norm this product follows (a layer used with another
+      // norm, or with none, gets its copy made again)
+      const float *gamma = qkv.norm ? qkv.gamma : nullptr;
+      if (gamma != l->w_qkv_t_gamma) l->w_qkv_t_stale = true;
+      qkv.w_t = transposed_twin(&l->w_qkv_t, &l->w_qkv_t_stale, l->w_qkv, l->d_model, wide, stream, gamma);
+      l->w_qkv_t_gamma = qkv.w_t ? gamma : nullptr;
+      qkv.w_t_has_gamma = qkv.w_t && gamma;
+    }
     if ((rc = l->proj.project(x, l->d_model, l->w_qkv, nullptr, T, l->d_model, wide, stream, qkv))) return rc;
     // One row: the attention launch leaves the memory system idle while it waits on its chain of
     // dependent loads, and takes along workgroups that read the first rows of the gate | up
@@ -337,7 +346,10 @@ int block_forward_device(shainet_llama_block *b, const float *x, int T, float *o
   gate.gamma = b->norm2;
   gate.eps = b->eps;
   gate.epilogue = kGemvSwiglu;
-  if (gemvt_takes(T, d, ff, gate.epilogue, true)) gate.w_t = transposed_twin(&b->gate_up_t, &b->gate_up_t_stale, b->gate_up, d, 2 * ff, stream);
+  if (gemvt_takes(T, d, ff, gate.epilogue, true)) {
+    gate.w_t = transposed_twin(&b->gate_up_t, &b->gate_up_t_stale, b->gate_up, d, 2 * ff, stream, b->norm2);
+    gate.w_t_has_gamma = gate.w_t && b->norm2;
+  }
   const AheadRows ahead = {gate.w_t, d, ff};
   if ((rc = attn_forward_device(l, x, T, b->h.p, n1, x, no_cache, &ahead))) return rc;
   // hidden = silu(normed2 * gate_proj) * (normed2 * up_proj), normed2 = @norm2.forward(h)
@@ -501,6 +513,9 @@ int shainet_llama_block_set_norms(shainet_llama_block *b, const float *norm1, co
       *dst[i] = nullptr;
     }
   }
+  // (the transposed copies of q | k | v and gate | up carry the norm weights)
+  b->attn->w_qkv_t_stale = b->gate_up_t_stale = true;
+  b->attn->w_qkv_t_gamma = nullptr;
   return rc;
 }
 

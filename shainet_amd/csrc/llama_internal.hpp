@@ -75,6 +75,7 @@ struct Fused {
   // the same weights transposed ([N, K]; kGemvSwiglu: [2N, K]) or null: one row of x then takes the
   // product that gives a wavefront whole outputs (launch_gemvt) where its shapes allow
   const float *w_t = nullptr;
+  bool w_t_has_gamma = false;  // the rows of w_t were made with gamma multiplied in: the norm's factor 1 / rms is all that is left to apply
 };
 
 // y[T,N] = epilogue(norm(x)[T,K] * W), all row-major on the device.  Up to 16 rows
@@ -117,6 +118,9 @@ int llama_fail(int code, const std::string &msg);
 // the device) transposed, allocated on first use and made again when *stale; returns the twin, or
 // null when they are turned off or there is no memory for one (the caller then goes without).
 bool transposed_twins_wanted();
-const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream);
+// row_scale (nullable): a factor per row of src, i.e. per input of the product: the RMSNorm weights
+// gamma of the norm the product always follows, so that (x gamma) W = x (diag(gamma) W) needs no gamma.
+const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream,
+                             const float *row_scale = nullptr);
 
 }  // namespace shainet

@@ -73,7 +73,8 @@ bool transposed_twins_wanted() {
 
 // *twin = src transposed (src: [rows, cols] on the device), allocated on first use.  Returns the
 // twin, or null when there is no memory for it (the caller then goes without).
-const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream) {
+const float *transposed_twin(float **twin, bool *stale, const float *src, int rows, int cols, hipStream_t stream,
+                             const float *row_scale) {
   if (!transposed_twins_wanted() || !src) return nullptr;
   if (!*twin) {
     if (hipMalloc((void **)twin, (size_t)rows * cols * sizeof(float)) != hipSuccess) {
@@ -85,7 +86,7 @@ const float *transposed_twin(float **twin, bool *stale, const float *src, int ro
   }
   if (*stale) {
     // (waited for, once per set of weights: the copy may next be read on another stream)
-    if (launch_transpose(src, *twin, rows, cols, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) {
+    if (launch_transpose(src, *twin, rows, cols, stream, row_scale) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) {
       (void)hipGetLastError();
       return nullptr;
     }
@@ -137,7 +138,7 @@ int Projector::project(const float *x, long long x_stride, const float *w, float
     a.x = x;
     a.x_stride = x_stride;
     a.norm = f.norm ? 1 : 0;
-    a.gamma = f.gamma;
+    a.gamma = f.w_t_has_gamma ? nullptr : f.gamma;
     a.eps = f.eps;
     a.w = f.w_t;
     a.res = f.res;

@@ -511,6 +511,10 @@ def test_single_row_products_over_transposed_weights(hip, tied, d, H, KV, ff):
     lw = w["layers"][1]
     lw["w_q"], lw["w_v"], lw["w_o"], lw["gate"], lw["down"] = g(d, H * hd), g(d, KV * hd), g(H * hd, d), g(d, ff), g(ff, d)
     m.blocks[1].set_weights(lw["w_q"], lw["w_k"], lw["w_v"], lw["w_o"]); m.blocks[1].set_ffn(lw["gate"], lw["up"], lw["down"])
+    # (and other norm weights in block 0: the copies of q | k | v and gate | up carry them)
+    l0 = w["layers"][0]
+    l0["norm1"], l0["norm2"] = ((1 + 0.2 * r.standard_normal(d)).astype(np.float32) for _ in range(2))
+    m.blocks[0].set_norms(l0["norm1"], l0["norm2"])
     w["lm_head"] = g(d, V)
     m.set_lm_head(w["lm_head"])
     om = tinyllama.OracleModel(w, orc)
