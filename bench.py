@@ -369,9 +369,11 @@ def model_decode(sa, np, steps, ctx_len=512):
     # one block's worth of seeded weights, uploaded into every block (timing does not depend on the values)
     ws = [(0.02 * r.standard_normal(sh, dtype=np.float32)) for sh in
           ((d, H * hd), (d, KV * hd), (d, KV * hd), (H * hd, d), (d, ff), (d, ff), (ff, d))]
+    gammas = [(1 + 0.1 * r.standard_normal(d)).astype(np.float32) for _ in range(2)]
     for b in m.blocks:
         b.set_weights(*ws[:4])
         b.set_ffn(*ws[4:])
+        b.set_norms(*gammas)  # (a Llama block has both norm weights)
     del ws
     weight_bytes = 4 * (L * (2 * d * H * hd + 2 * d * KV * hd + 3 * d * ff) + d * V)
     # prefill of the context: more than 16 rows go through the library's own MFMA product and the MFMA attention kernel
