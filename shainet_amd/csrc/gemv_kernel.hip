@@ -466,24 +466,28 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   constexpr int XC = KV4 < 8 ? KV4 : 8;
   const float *xp = a.x + seg * KW + 4 * lane;
   float *my_xs = xs + (XLDS ? wave * KW : 0) + 4 * lane;
-  double rms = 1.0;  // 1 / the root mean square
+  float rms = 1.0f;  // 1 / the root mean square
   if (a.norm) {
-    // every wavefront of the launch runs this: a lane's 4 KV4 squares are added up in fp32 (fp64
-    // sums cost 0.4 us of a 3072-row product), the lanes' sums, the mean and the root in fp64
-    double sq = 0.0;
+    // every wavefront of the launch runs this, so it is kept short: squares, their sums and the
+    // root in fp32 (a reciprocal square root and one Newton step; all of it in fp64 as
+    // rms_norm.cr does cost 0.4 us of a 3072-row product for the sums and as much for the root);
+    // the factor is within a few 1e-7 of the fp64 one
+    f32x4 q = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c0 = 0; c0 < KV4; c0 += XC) {
       f32x4 t[XC];
 #pragma unroll
       for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
-      f32x4 q = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < XC; ++i) q += t[i] * t[i];
-      sq += (double)((q.x + q.y) + (q.z + q.w));
     }
+    float sq = (q.x + q.y) + (q.z + q.w);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
-    rms = 1.0 / sqrt(sq / (double)K + a.eps);
+    const float m = sq / (float)K + (float)a.eps;
+    float r = rsqrtf(m);
+    r = r * (1.5f - 0.5f * m * r * r);
+    rms = r;
   }
   // pieces c0 .. c0 + XC - 1 of x, normed if asked
   auto x_pieces = [&](f32x4 (&t)[XC], int c0) {
@@ -551,7 +555,7 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     }
     if (a.norm) {
 #pragma unroll
-      for (int c = 0; c < NACC; ++c) s[c] = (float)((double)s[c] * rms);
+      for (int c = 0; c < NACC; ++c) s[c] = s[c] * rms;
     }
     if constexpr (PREP) {
       if (lane == 0) half_s[wave] = s[0];
