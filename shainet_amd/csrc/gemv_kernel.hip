@@ -444,11 +444,12 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   // (with SP = 2 both wavefronts of a pair see the same n0: they leave together)
   if (!PREP && !live) return;
   const int half_hd = PREP ? a.prep.hd >> 1 : 1;
+  const int half_shift = PREP ? __builtin_ctz(half_hd) : 0;
   const int upper = PREP ? wave >> 1 : 0;
   auto load_row = [&](f32x4 (&w)[NACC][KV4], int n) {
 #pragma unroll
     for (int c = 0; c < NACC; ++c) {
-      const long long wrow = PREP ? (long long)n + (n / half_hd + upper) * half_hd : (long long)c * N + n;
+      const long long wrow = PREP ? (long long)n + (((n >> half_shift) + upper) << half_shift) : (long long)c * N + n;
       const float *row = a.w + wrow * K + seg * KW + 4 * lane;
 #pragma unroll
       for (int i = 0; i < KV4; ++i) w[c][i] = __builtin_nontemporal_load((const f32x4 *)(row + 256 * i));
@@ -461,12 +462,18 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   float res_first = 0.f;
   if (residual) res_first = a.res[n0];
   PairTarget target = {};
-  if constexpr (PREP) target = prep_pair_begin(a.prep, n0 / half_hd, n0 % half_hd);
+  // (head_dim is a power of two here: gemvt_takes)
+  if constexpr (PREP) target = prep_pair_begin(a.prep, n0 >> half_shift, n0 & (half_hd - 1));
 
   constexpr int XC = KV4 < 8 ? KV4 : 8;
   const float *xp = a.x + seg * KW + 4 * lane;
   float *my_xs = xs + (XLDS ? wave * KW : 0) + 4 * lane;
   float rms = 1.0f;  // 1 / the root mean square
+  f32x4 xv[XREG ? KV4 : 1];
+  if constexpr (XREG) {  // x is loaded once, into the registers it stays in
+#pragma unroll
+    for (int i = 0; i < KV4; ++i) xv[i] = *(const f32x4 *)(xp + 256 * i);
+  }
   if (a.norm) {
     // every wavefront of the launch runs this, so it is kept short: squares, their sums and the
     // root in fp32 (a reciprocal square root and one Newton step; all of it in fp64 as
@@ -477,7 +484,7 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     for (int c0 = 0; c0 < KV4; c0 += XC) {
       f32x4 t[XC];
 #pragma unroll
-      for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
+      for (int i = 0; i < XC; ++i) t[i] = XREG ? xv[c0 + i] : *(const f32x4 *)(xp + 256 * (c0 + i));
 #pragma unroll
       for (int i = 0; i < XC; ++i) q += t[i] * t[i];
     }
@@ -502,19 +509,18 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       }
     }
   };
-  f32x4 xv[XREG ? KV4 : 1];
-  if constexpr (XREG || XLDS) {
+  if constexpr (XREG) {
+    if (a.norm && a.gamma) {
+#pragma unroll
+      for (int i = 0; i < KV4; ++i) xv[i] = xv[i] * *(const f32x4 *)(a.gamma + 4 * lane + 256 * i);
+    }
+  } else if constexpr (XLDS) {
 #pragma unroll
     for (int c0 = 0; c0 < KV4; c0 += XC) {
       f32x4 t[XC];
       x_pieces(t, c0);
 #pragma unroll
-      for (int i = 0; i < XC; ++i) {
-        if constexpr (XREG)
-          xv[c0 + i] = t[i];
-        else
-          *(f32x4 *)(my_xs + 256 * (c0 + i)) = t[i];  // read back by this lane only: no barrier
-      }
+      for (int i = 0; i < XC; ++i) *(f32x4 *)(my_xs + 256 * (c0 + i)) = t[i];  // read back by this lane only: no barrier
     }
   }
 
@@ -681,7 +687,7 @@ hipError_t launch_gemv(const GemvArgs &args, const GemvPlan &p, hipStream_t stre
 bool gemvt_takes(int T, int K, int N, int epilogue, bool norm, const GemvPrep *prep) {
   if (T != 1 || N < 1) return false;
   if (epilogue == kGemvQkvPrep) {
-    if (!prep || prep->q_norm || prep->k_norm || prep->hd < 2 || (prep->hd & 1)) return false;
+    if (!prep || prep->q_norm || prep->k_norm || prep->hd < 2 || (prep->hd & (prep->hd - 1))) return false;
     return (K == 1024 || K == 2048 || K == 4096) && N == (prep->H + 2 * prep->KV) * prep->hd;
   }
   // rows of 8192: two wavefronts per output, which leaves out the norm prologue and SwiGLU
