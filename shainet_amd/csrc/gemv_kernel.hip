@@ -427,8 +427,13 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   // x: up to 2048 values stay in registers.  Longer (half) rows: a wavefront with one output reads
   // them again from memory (the L2), eight 16-byte pieces at a time, where they are used; one with
   // several outputs keeps its own normed copy in LDS
-  constexpr bool XREG = KV4 <= 8, XLDS = !XREG && MULTI;
+  // Rows of 8192 with one output per pair of wavefronts: the workgroup puts x into LDS once, asked
+  // for before the weights (read piece by piece from the L2 where it is used, x came back behind
+  // the weight loads it was issued after, a round trip at the end of every wavefront, and the
+  // registers for it left room for two wavefronts per SIMD)
+  constexpr bool XREG = KV4 <= 8, XLDS = !XREG && MULTI, XSH = SP == 2 && !MULTI;
   __shared__ __align__(16) float xs[XLDS ? 4 * 256 * KV4 : 4];
+  __shared__ __align__(16) float xsh[XSH ? 256 * KV4 * SP : 4];
   __shared__ float half_s[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rpw = a.rows_per_wave;
@@ -456,7 +461,17 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     }
   };
   f32x4 wa[NACC][KV4], wb[MULTI ? NACC : 1][MULTI ? KV4 : 1];
+  f32x4 x_own[XSH ? K / 1024 : 1];  // this thread's share of x on its way to LDS
+  if constexpr (XSH) {
+#pragma unroll
+    for (int i = 0; i < K / 1024; ++i) x_own[i] = *(const f32x4 *)(a.x + 4 * threadIdx.x + 1024 * i);
+  }
   load_row(wa, n0);
+  if constexpr (XSH) {
+#pragma unroll
+    for (int i = 0; i < K / 1024; ++i) *(f32x4 *)(xsh + 4 * threadIdx.x + 1024 * i) = x_own[i];
+    __syncthreads();
+  }
   // what the epilogue of the first output reads besides: asked for now, behind the weights
   const bool residual = !PREP && a.epilogue == kGemvResidual;
   float res_first = 0.f;
@@ -537,6 +552,9 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       } else if constexpr (XLDS) {
 #pragma unroll
         for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(my_xs + 256 * (c0 + i));
+      } else if constexpr (XSH) {
+#pragma unroll
+        for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xsh + seg * KW + 4 * lane + 256 * (c0 + i));
       } else {
         x_pieces(t, c0);
       }
