@@ -427,14 +427,16 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   // x: up to 2048 values stay in registers.  Longer (half) rows: a wavefront with one output reads
   // them again from memory (the L2), eight 16-byte pieces at a time, where they are used; one with
   // several outputs keeps its own normed copy in LDS
-  // Rows of 8192 with one output per pair of wavefronts: the workgroup puts x into LDS once, asked
-  // for before the weights (read piece by piece from the L2 where it is used, x came back behind
-  // the weight loads it was issued after, a round trip at the end of every wavefront, and the
-  // registers for it left room for two wavefronts per SIMD)
-  constexpr bool XREG = KV4 <= 8, XLDS = !XREG && MULTI, XSH = SP == 2 && !MULTI;
+  // One output per wavefront (XSH): the workgroup puts x into LDS once, asked for before the
+  // weights, each thread a share of it; the share's squares give the norm's sum once per workgroup
+  // (rows of 8192 first: read piece by piece from the L2 where it was used, x came back behind the
+  // weight loads it was issued after, a round trip at the end of every wavefront, and the
+  // registers for it left room for two wavefronts per SIMD).  Several outputs per wavefront:
+  // x in registers (XREG) or a normed copy per wavefront in LDS (XLDS), as described above.
+  constexpr bool XSH = !MULTI, XREG = !XSH && KV4 <= 8, XLDS = !XSH && !XREG;
   __shared__ __align__(16) float xs[XLDS ? 4 * 256 * KV4 : 4];
   __shared__ __align__(16) float xsh[XSH ? 256 * KV4 * SP : 4];
-  __shared__ float half_s[4];
+  __shared__ float half_s[4], sq_s[4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rpw = a.rows_per_wave;
   const int N = a.N;
@@ -446,8 +448,9 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   const int seg = wave % SP;
   constexpr int KW = 256 * KV4;  // values per wavefront and row
   constexpr int K = KW * SP;
-  // (with SP = 2 both wavefronts of a pair see the same n0: they leave together)
-  if (!PREP && !live) return;
+  // (with SP = 2 both wavefronts of a pair see the same n0: they are live or not together; XSH:
+  // wavefronts without an output stay for the workgroup's x and leave after its barrier)
+  if (!PREP && !XSH && !live) return;
   const int half_hd = PREP ? a.prep.hd >> 1 : 1;
   const int half_shift = PREP ? __builtin_ctz(half_hd) : 0;
   const int upper = PREP ? wave >> 1 : 0;
@@ -461,16 +464,43 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     }
   };
   f32x4 wa[NACC][KV4], wb[MULTI ? NACC : 1][MULTI ? KV4 : 1];
-  f32x4 x_own[XSH ? K / 1024 : 1];  // this thread's share of x on its way to LDS
+  float rms = 1.0f;  // 1 / the root mean square
+  constexpr bool NORMS = SP == 1;  // (rows shared by two wavefronts come without the norm: gemvt_takes)
+  f32x4 x_own[XSH ? K / 1024 : 1], g_own[XSH && NORMS ? K / 1024 : 1];  // this thread's share of x (and gamma) on its way to LDS
   if constexpr (XSH) {
 #pragma unroll
     for (int i = 0; i < K / 1024; ++i) x_own[i] = *(const f32x4 *)(a.x + 4 * threadIdx.x + 1024 * i);
+    if (NORMS && a.norm && a.gamma) {
+#pragma unroll
+      for (int i = 0; i < K / 1024; ++i) g_own[i] = *(const f32x4 *)(a.gamma + 4 * threadIdx.x + 1024 * i);
+    }
   }
-  load_row(wa, n0);
+  if (live || PREP) load_row(wa, n0);
   if constexpr (XSH) {
+    if (NORMS && a.norm) {
+      // squares, their sums and the root in fp32 (a reciprocal square root and one Newton step):
+      // within a few 1e-7 of the fp64 factor of rms_norm.cr:18-37
+      f32x4 q = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < K / 1024; ++i) q += x_own[i] * x_own[i];
+      float sq = (q.x + q.y) + (q.z + q.w);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+      if (lane == 0) sq_s[wave] = sq;
+      if (a.gamma) {
+#pragma unroll
+        for (int i = 0; i < K / 1024; ++i) x_own[i] = x_own[i] * g_own[i];  // (1 / rms multiplies the finished sum)
+      }
+    }
 #pragma unroll
     for (int i = 0; i < K / 1024; ++i) *(f32x4 *)(xsh + 4 * threadIdx.x + 1024 * i) = x_own[i];
     __syncthreads();
+    if (!PREP && !live) return;
+    if (NORMS && a.norm) {
+      const float m = ((sq_s[0] + sq_s[1]) + (sq_s[2] + sq_s[3])) / (float)K + (float)a.eps;
+      float r = rsqrtf(m);
+      rms = r * (1.5f - 0.5f * m * r * r);
+    }
   }
   // what the epilogue of the first output reads besides: asked for now, behind the weights
   const bool residual = !PREP && a.epilogue == kGemvResidual;
@@ -483,13 +513,12 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
   constexpr int XC = KV4 < 8 ? KV4 : 8;
   const float *xp = a.x + seg * KW + 4 * lane;
   float *my_xs = xs + (XLDS ? wave * KW : 0) + 4 * lane;
-  float rms = 1.0f;  // 1 / the root mean square
   f32x4 xv[XREG ? KV4 : 1];
   if constexpr (XREG) {  // x is loaded once, into the registers it stays in
 #pragma unroll
     for (int i = 0; i < KV4; ++i) xv[i] = *(const f32x4 *)(xp + 256 * i);
   }
-  if (a.norm) {
+  if (!XSH && a.norm) {
     // every wavefront of the launch runs this, so it is kept short: squares, their sums and the
     // root in fp32 (a reciprocal square root and one Newton step; all of it in fp64 as
     // rms_norm.cr does cost 0.4 us of a 3072-row product for the sums and as much for the root);
