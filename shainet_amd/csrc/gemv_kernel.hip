@@ -540,7 +540,7 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
     r = r * (1.5f - 0.5f * m * r * r);
     rms = r;
   }
-  // pieces c0 .. c0 + XC - 1 of x, normed if asked
+  // pieces c0 .. c0 + XC - 1 of x times gamma (for the copy of XLDS)
   auto x_pieces = [&](f32x4 (&t)[XC], int c0) {
 #pragma unroll
     for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xp + 256 * (c0 + i));
@@ -581,11 +581,9 @@ __global__ __launch_bounds__(256) void gemvt_kernel(GemvArgs a) {
       } else if constexpr (XLDS) {
 #pragma unroll
         for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(my_xs + 256 * (c0 + i));
-      } else if constexpr (XSH) {
+      } else {  // XSH
 #pragma unroll
         for (int i = 0; i < XC; ++i) t[i] = *(const f32x4 *)(xsh + seg * KW + 4 * lane + 256 * (c0 + i));
-      } else {
-        x_pieces(t, c0);
       }
 #pragma unroll
       for (int c = 0; c < NACC; ++c)
